@@ -173,8 +173,9 @@ class CachePools:
             for i, cache_id in enumerate(gl.buffers):
                 self.index[cache_id] = (g, i)
         # one slot more than requests can hold: the padded rows of a recorded step are pointed at it
-        self.state = {cid: torch.zeros((num_state_slots + 1,) + tuple(st.shape), dtype=st.dtype, device=device)
-                      for cid, st in layout.states.items()}
+        # keys: a cache id for a mixer's state, (cache id, name) for another part's (Block.state_specs)
+        self.state = {cid: torch.zeros((num_state_slots + 1,) + tuple(st.shape), dtype=st.dtype or dtype, device=device)
+                      for cid, st in {**layout.states, **layout.part_states}.items()}
 
     def buffer(self, cache_id: int):
         """-> (group, {page tensor name: [pages, *page shape]}) of one cache buffer."""

@@ -3,7 +3,7 @@
 ``ARCHITECTURES`` maps the string in config.json's ``architectures`` list to an
 architecture (a typed configuration class plus a function that turns such a
 configuration into a ``ModelSpec``).  ``MIXERS``, ``FEED_FORWARDS``, ``NORMS``,
-``POSITION_ENCODINGS``, ``BLOCKS``, ``EMBEDDINGS`` and ``HEADS`` map a
+``POSITION_ENCODINGS``, ``BLOCKS``, ``EMBEDDINGS``, ``HEADS``, ``FILTERS`` and ``STREAM_SHIFTS`` map a
 ``PartSpec.kind`` to a part class.
 Code outside this package (a test, a plug-in) adds an entry with
 ``@REGISTRY.register("name")`` and needs no change to the package's files.
@@ -68,6 +68,8 @@ POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("output head")
+FILTERS = Registry("input filter")
+STREAM_SHIFTS = Registry("stream shift")
 
 
 def register_architecture(name: str, config_class: Any, to_spec: Callable[[Any], Any], *, replace: bool = False):
@@ -78,6 +80,8 @@ def architecture_of(config_dict: dict) -> Architecture:
     """The architecture a config.json asks for: the first name of its
     ``architectures`` list that is registered."""
     names = config_dict.get("architectures")
+    if not names and isinstance(config_dict.get("architecture"), str):
+        names = [config_dict["architecture"]]      # files that name their one architecture in the singular
     if not names:
         raise KeyError(f"config.json has no 'architectures' entry; known: {ARCHITECTURES.names()}")
     for n in names:

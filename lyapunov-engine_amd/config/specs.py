@@ -13,7 +13,7 @@ filled.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Mapping
+from typing import Mapping, Optional
 
 
 @dataclass(frozen=True)
@@ -29,7 +29,7 @@ class PartSpec:
 class LayerSpec:
     block: str                      # arrangement of the parts, e.g. "prenorm"
     mixer: PartSpec
-    ffn: PartSpec
+    ffn: Optional[PartSpec]         # None: the layer has no feed-forward branch (for arrangements that allow it)
     norm1: PartSpec                 # before the mixer
     norm2: PartSpec                 # before the feed-forward
     # Names of the four parts inside the layer's tensor-name prefix ("norm1", "mixer", "norm2",
@@ -41,6 +41,8 @@ class LayerSpec:
     # kind decides which registry each comes from and what its tensors are
     # called.  "prenorm" takes none.
     extra: Mapping = field(default_factory=dict)
+    # Constants of the arrangement itself (a multiplier on what joins the stream, ...): name -> number.
+    params: Mapping = field(default_factory=dict)
 
     def __post_init__(self):
         missing = [k for k in ("norm1", "mixer", "norm2", "ffn") if k not in self.names]
@@ -59,12 +61,15 @@ class LayerCall:
     ``cache``   which cache buffer its mixer uses; calls that name the same
                 buffer share keys and values;
     ``writes``  false: the mixer only reads the buffer (another call filled it)
-                and computes no keys and values of its own.
+                and computes no keys and values of its own;
+    ``shift``   a row of the model's stream shift (``ModelSpec.stream_shift``)
+                that is added to the residual stream right before this call.
     """
 
     layer: int
     cache: int
     writes: bool = True
+    shift: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -87,6 +92,10 @@ class ModelSpec:
     layer_prefix: str                # with "{i}" for the layer's number
     embedding: PartSpec = PartSpec("lookup")
     head: PartSpec = PartSpec("linear")
+    # A table of vectors of which calls of the running order add one to the residual stream
+    # (``LayerCall.shift``), and the tensor-name prefix it is found under.
+    stream_shift: Optional[PartSpec] = None
+    stream_shift_prefix: str = ""
     eos_token_ids: tuple = ()
     ignorable_tensors: tuple = ()    # shell-style patterns of tensor names a file may hold unused
     init_std: float = 0.02           # random-weights mode: normal(0, init_std) matrices

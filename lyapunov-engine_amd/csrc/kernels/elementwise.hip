@@ -19,11 +19,11 @@ namespace lyp {
 // ------------------------------------------------------------------ embedding
 template <typename TW>
 __global__ void embedding_kernel(const int32_t* __restrict__ ids, const TW* __restrict__ table,
-                                 float* __restrict__ out, int H) {
+                                 float* __restrict__ out, int H, float scale) {
   const int t = blockIdx.x;
   const TW* row = table + static_cast<size_t>(ids[t]) * H;
   float* o = out + static_cast<size_t>(t) * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32(row[i]);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32(row[i]) * scale;
 }
 
 // -------------------------------------------------------------------- RMSNorm
@@ -479,15 +479,15 @@ int lyp_table_load(const int32_t* src, int32_t* dst, int n, const int32_t* patch
   return 0;
 }
 
-int lyp_embedding(const int32_t* ids, const void* table, int table_dtype, float* out, int T, int H,
+int lyp_embedding(const int32_t* ids, const void* table, int table_dtype, float* out, int T, int H, float scale,
                   hipStream_t stream) {
   LYP_REQUIRE(T >= 0 && H > 0, "embedding: bad sizes T=%d H=%d", T, H);
   if (T == 0) return 0;
   const int threads = H >= 1024 ? 256 : 128;
   if (table_dtype == kF32)
-    embedding_kernel<float><<<T, threads, 0, stream>>>(ids, static_cast<const float*>(table), out, H);
+    embedding_kernel<float><<<T, threads, 0, stream>>>(ids, static_cast<const float*>(table), out, H, scale);
   else if (table_dtype == kBF16)
-    embedding_kernel<bf16_t><<<T, threads, 0, stream>>>(ids, static_cast<const bf16_t*>(table), out, H);
+    embedding_kernel<bf16_t><<<T, threads, 0, stream>>>(ids, static_cast<const bf16_t*>(table), out, H, scale);
   else
     LYP_REQUIRE(false, "embedding: unknown table dtype %d", table_dtype);
   LYP_LAUNCH_CHECK("embedding");

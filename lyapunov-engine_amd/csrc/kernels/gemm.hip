@@ -42,8 +42,14 @@ template <typename T, int BM, int BN, int WGM, int WGN, int MODE>
 __global__ __launch_bounds__(256) void gemm_nt_kernel(const T* __restrict__ A,
                                                       const T* __restrict__ W, void* __restrict__ Cv,
                                                       int M, int N, int K, int lda, int ldw, int ldc,
-                                                      int vec_ok) {
+                                                      int vec_ok, long long batch_a = 0, long long batch_w = 0,
+                                                      long long batch_c = 0) {
   static_assert(WGM * WGN == 4, "four waves per workgroup");
+  // blockIdx.z: one of several products of equal shape whose operands lie batch_* elements apart
+  A += blockIdx.z * batch_a;
+  W += blockIdx.z * batch_w;
+  if constexpr (MODE == kStoreAct) Cv = static_cast<T*>(Cv) + blockIdx.z * batch_c;
+  else Cv = static_cast<float*>(Cv) + blockIdx.z * batch_c;
   constexpr int VEC = VecOf<T>::kVec;
   constexpr int KF = Mma32<T>::kElems;
   constexpr int PAD = VEC;
@@ -1041,6 +1047,48 @@ using namespace lyp;
 extern "C" int lyp_gemm_wide(int which) {
   LYP_REQUIRE(which >= 0 && which <= 3, "wide product: 0 to 3, not %d", which);
   g_wide_gemm = which;
+  return 0;
+}
+
+// `batch` products of one shape in one launch of the tiled kernel: product z reads A + z * batch_a
+// and W + z * batch_w and writes C + z * batch_c (in elements; heads that lie side by side in the
+// rows of one tensor, each with a matrix of its own).
+extern "C" int lyp_gemm_nt_batched(const void* A, const void* W, void* C, int dtype, int mode, int batch, int M, int N,
+                                   int K, int lda, int ldw, int ldc, long long batch_a, long long batch_w,
+                                   long long batch_c, hipStream_t stream) {
+  LYP_REQUIRE(M >= 0 && N > 0 && K > 0 && batch > 0 && batch <= 65535, "batched gemm: bad sizes batch=%d M=%d N=%d K=%d",
+              batch, M, N, K);
+  LYP_REQUIRE(lda >= K && ldw >= K && ldc >= N, "batched gemm: leading dimensions %d %d %d too small", lda, ldw, ldc);
+  LYP_REQUIRE(mode == kStoreAct || mode == kStoreF32, "batched gemm: output mode %d", mode);
+  LYP_REQUIRE((M + 127) / 128 <= 65535, "batched gemm: M=%d too large for one launch", M);
+  if (M == 0) return 0;
+  const int vec = dtype == kF32 ? 4 : 8;
+  const int vec_ok = (lda % vec == 0) && (ldw % vec == 0) && (batch_a % vec == 0) && (batch_w % vec == 0) &&
+                     (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(W) % 16 == 0);
+#define LYP_BGEMM(T, MODE)                                                                                     \
+  do {                                                                                                         \
+    const T* a_ = static_cast<const T*>(A);                                                                    \
+    const T* w_ = static_cast<const T*>(W);                                                                    \
+    if (M <= 32) {                                                                                             \
+      dim3 grid((N + 127) / 128, (M + 31) / 32, batch);                                                        \
+      gemm_nt_kernel<T, 32, 128, 1, 4, MODE><<<grid, 256, 0, stream>>>(a_, w_, C, M, N, K, lda, ldw, ldc,      \
+                                                                       vec_ok, batch_a, batch_w, batch_c);     \
+    } else if (M <= 64) {                                                                                      \
+      dim3 grid((N + 127) / 128, (M + 63) / 64, batch);                                                        \
+      gemm_nt_kernel<T, 64, 128, 2, 2, MODE><<<grid, 256, 0, stream>>>(a_, w_, C, M, N, K, lda, ldw, ldc,      \
+                                                                       vec_ok, batch_a, batch_w, batch_c);     \
+    } else {                                                                                                   \
+      dim3 grid((N + 127) / 128, (M + 127) / 128, batch);                                                      \
+      gemm_nt_kernel<T, 128, 128, 2, 2, MODE><<<grid, 256, 0, stream>>>(a_, w_, C, M, N, K, lda, ldw, ldc,     \
+                                                                        vec_ok, batch_a, batch_w, batch_c);    \
+    }                                                                                                          \
+  } while (0)
+  if (dtype == kF32) LYP_BGEMM(float, kStoreF32);
+  else if (dtype == kBF16 && mode == kStoreAct) LYP_BGEMM(bf16_t, kStoreAct);
+  else if (dtype == kBF16) LYP_BGEMM(bf16_t, kStoreF32);
+  else LYP_REQUIRE(false, "batched gemm: unknown dtype %d", dtype);
+#undef LYP_BGEMM
+  LYP_LAUNCH_CHECK("gemm_nt_batched");
   return 0;
 }
 

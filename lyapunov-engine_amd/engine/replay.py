@@ -14,7 +14,7 @@ import numpy as np
 
 from .core import EngineCore, StepEntry
 
-MAX_LIVE_REQUESTS = 8
+MAX_LIVE_REQUESTS = 4
 
 
 class TraceReplayer:

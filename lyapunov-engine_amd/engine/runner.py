@@ -114,7 +114,8 @@ class ModelRunner:
         for call in model.schedule:
             g = self.layout.group_of(call.cache)
             pages = pools.buffer(call.cache)[1] if g is not None else {}
-            self._calls.append((g, pages, pools.state.get(call.cache), call.writes))
+            further = {name: pools.state[(cid, name)] for cid, name in self.layout.part_states if cid == call.cache}
+            self._calls.append((g, pages, pools.state.get(call.cache), call.writes, further))
         # the parts' planners, one per distinct key, in the order the parts come
         self.planners: dict = {}
         for _, part in model.named_parts():
@@ -309,8 +310,9 @@ class ModelRunner:
         return self.context(tables, dev)
 
     def layer_caches(self, ctx: StepContext) -> list:
-        return [LayerCache(group=ctx.groups[g] if g is not None else None, pages=pages, state=state, writes=writes)
-                for g, pages, state, writes in self._calls]
+        return [LayerCache(group=ctx.groups[g] if g is not None else None, pages=pages, state=state, writes=writes,
+                           states=further)
+                for g, pages, state, writes, further in self._calls]
 
     # --------------------------------------------------------------- the step
     def step(self, entries: list) -> Optional[torch.Tensor]:

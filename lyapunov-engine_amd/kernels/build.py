@@ -36,7 +36,8 @@ HIP_FLAGS = [
 ]
 CXX_FLAGS = ["-O2", "-std=c++20", "-fPIC", "-Wall", "-Wextra"]
 
-CORE_SOURCES = ["kernels/errors.hip", "kernels/elementwise.hip", "kernels/gemm.hip", "kernels/sampler.hip"]
+CORE_SOURCES = ["kernels/errors.hip", "kernels/elementwise.hip", "kernels/sequence.hip", "kernels/gemm.hip",
+                "kernels/sampler.hip"]
 ATTN_SOURCES = ["kernels/errors.hip", "kernels/attention.hip"]
 BLAS_SOURCES = ["kernels/errors.hip", "kernels/library_gemm.hip"]   # host code around the vendor's GEMM library
 RUNTIME_SOURCES = ["runtime/cache_manager.cpp", "runtime/scheduler.cpp", "runtime/c_api.cpp"]

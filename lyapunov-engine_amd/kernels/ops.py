@@ -43,7 +43,7 @@ def core() -> ctypes.CDLL:
     if _core is None:
         lib = _load(build.core_library())
         lib.lyp_last_error.restype = ctypes.c_char_p
-        lib.lyp_embedding.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p]
+        lib.lyp_embedding.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]
         lib.lyp_table_load.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p]
         lib.lyp_rmsnorm.argtypes = [c_void_p, c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p, c_int, c_void_p,
                                     c_int, c_int, c_float, c_void_p]
@@ -86,6 +86,23 @@ def core() -> ctypes.CDLL:
         lib.lyp_skinny_slices.argtypes = [c_int, c_int]
         lib.lyp_stream_read.argtypes = [c_void_p, c_longlong, c_int, c_void_p, c_void_p]
         lib.lyp_stream_rows.argtypes = [c_void_p, c_longlong, c_int, c_int, c_int, c_void_p, c_void_p]
+        lib.lyp_gemm_nt_batched.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                            c_int, c_int, c_int, c_longlong, c_longlong, c_longlong, c_void_p]
+        lib.lyp_branch_join.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
+                                        c_int, c_void_p, c_int, c_int, c_float, c_float, c_void_p]
+        lib.lyp_add_row.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p]
+        lib.lyp_short_conv.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                       c_int, c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_activation.argtypes = [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p, c_void_p]
+        lib.lyp_mingru_scan.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int, c_int, c_int, c_void_p]
+        lib.lyp_latent_prep.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]
+        lib.lyp_latent_query_rotate.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                                                c_int, c_int, c_int, c_void_p]
+        lib.lyp_latent_attn_rows.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                             c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                             c_void_p]
         _core = lib
     return _core
 
@@ -159,14 +176,14 @@ def _code(dt: torch.dtype) -> int:
 
 
 # ------------------------------------------------------------------ row kernels
-def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t, :] = table[ids[t], :] as float (the residual stream)."""
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] * scale as float (the residual stream)."""
     _dev(ids, table, out)
     T, H = out.shape
     if ids.dtype != torch.int32 or ids.numel() != T or table.shape[1] != H or out.dtype != torch.float32:
         raise KernelError(f"embedding: ids {tuple(ids.shape)} {ids.dtype}, table {tuple(table.shape)}, out {tuple(out.shape)} {out.dtype}")
     lib = core()
-    _check(lib.lyp_embedding(_p(ids), _p(table), _code(table.dtype), _p(out), T, H, _stream()), lib)
+    _check(lib.lyp_embedding(_p(ids), _p(table), _code(table.dtype), _p(out), T, H, float(scale), _stream()), lib)
     return out
 
 
@@ -210,6 +227,35 @@ class PendingNorm:
     def run(self) -> torch.Tensor:
         out = torch.empty(self.h.shape, dtype=self.dtype, device=self.h.device)
         return rmsnorm(self.h, self.weight, self.eps, out)
+
+
+class JoiningBranch:
+    """A branch's output that passes a norm of its own and a multiplier on its way into the residual
+    stream: h += mult * rmsnorm(y) * weight (+ shift, a vector for every row).  The norm that follows
+    (one with ``joins_branches``) does the sum in its own kernel; ``join(h)`` does it alone.
+    ``y`` [T, H] is in the activations' type or float, ``weight`` and ``shift`` are float."""
+
+    def __init__(self, y: torch.Tensor, weight: torch.Tensor, eps: float, mult: float = 1.0,
+                 shift: torch.Tensor | None = None):
+        self.y, self.weight, self.eps, self.mult, self.shift = y, weight, float(eps), float(mult), shift
+        self.shape = y.shape
+
+    def join(self, h: torch.Tensor) -> None:
+        """Carry the sum out on h; nothing is left to add (returns None)."""
+        branch_join(h, self.y, self.weight, self.mult, self.eps, shift=self.shift)
+        return None
+
+
+def shifted(h: torch.Tensor, delta, v: torch.Tensor):
+    """The residual stream h with what is still to be added to it (``delta``), plus the vector v on
+    every row.  A branch that is about to join takes v along; otherwise v is added to h now.
+    Returns what is still to be added."""
+    if isinstance(delta, JoiningBranch):
+        if delta.shift is None:
+            return JoiningBranch(delta.y, delta.weight, delta.eps, delta.mult, v)
+        delta = delta.join(h)
+    add_row(h, v)
+    return delta
 
 
 def as_delta(delta, dtype: torch.dtype):
@@ -772,6 +818,183 @@ def sum_parts(parts: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     out = torch.empty(parts.shape[1:], dtype=dtype, device=parts.device)
     lib = core()
     _check(lib.lyp_sum_parts(_p(parts), parts.shape[0], out.numel(), _p(out), _code(dtype), _stream()), lib)
+    return out
+
+
+def gemm_nt_heads(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[:, g, :] = a[:, g, :] @ w[g].T for every head g in one launch: a [M, G, K], w [G, N, K],
+    out [M, G, N] of a's dtype or float; views into wider tensors are fine as long as the last
+    dimension's values are neighbours."""
+    M, G, K = a.shape
+    N = w.shape[1]
+    if tuple(w.shape) != (G, N, K) or tuple(out.shape) != (M, G, N) or a.dtype != w.dtype or \
+            out.dtype not in (a.dtype, torch.float32):
+        raise KernelError(f"gemm_nt_heads: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, out {tuple(out.shape)}")
+    for name, t in (("a", a), ("w", w), ("out", out)):
+        if not t.is_cuda or t.stride(2) != 1:
+            raise KernelError(f"gemm_nt_heads: {name} {tuple(t.shape)} with strides {t.stride()} on {t.device}")
+    mode = STORE_ACT if out.dtype == a.dtype else STORE_F32
+    lib = core()
+    _check(lib.lyp_gemm_nt_batched(_p(a), _p(w), _p(out), _code(a.dtype), mode, G, M, N, K, a.stride(0), w.stride(1),
+                                   out.stride(0), a.stride(1), w.stride(0), out.stride(1), _stream()), lib)
+    return out
+
+
+# ------------------------------------------- branches with norms, filters, recurrences
+def _f32(*ts) -> None:
+    for t in ts:
+        if t is not None and t.dtype != torch.float32:
+            raise KernelError(f"small parameter vectors are kept in float32, got {t.dtype}")
+
+
+def branch_join(h: torch.Tensor, y: torch.Tensor | None, branch_weight: torch.Tensor | None, mult: float,
+                eps_branch: float, *, shift: torch.Tensor | None = None, next_weight: torch.Tensor | None = None,
+                eps_next: float = 0.0, out: torch.Tensor | None = None, rows: torch.Tensor | None = None):
+    """h += mult * rmsnorm(y) * branch_weight (+ shift, a vector added to every row), in 32-bit on the
+    residual stream; with ``next_weight`` the sum's RMS norm times that weight goes to ``out``
+    (activations).  ``rows`` picks the rows to join and norm into ``out`` and leaves h alone.
+    y [T, H] in the activations' type or float; None: only shift and norm."""
+    _dev(h, y, branch_weight, shift, next_weight, out, rows)
+    _f32(branch_weight, shift, next_weight)
+    T, H = h.shape
+    n = T if rows is None else rows.numel()
+    if h.dtype != torch.float32 or (y is not None and (tuple(y.shape) != (T, H) or branch_weight is None or
+                                                       branch_weight.numel() != H)):
+        raise KernelError(f"branch_join: h {tuple(h.shape)} {h.dtype}, y {None if y is None else tuple(y.shape)}")
+    if (shift is not None and shift.numel() != H) or (next_weight is not None and next_weight.numel() != H):
+        raise KernelError("branch_join: shift and the following norm's weights have one value per feature")
+    if next_weight is not None and (out is None or tuple(out.shape) != (n, H)):
+        raise KernelError("branch_join: the following norm needs an output of one row per joined row")
+    if rows is not None and (rows.dtype != torch.int32 or next_weight is None):
+        raise KernelError("branch_join: rows are int32 and only picked for a following norm")
+    lib = core()
+    _check(lib.lyp_branch_join(_p(h), _p(y), _code(y.dtype) if y is not None else 0, _p(branch_weight), float(mult),
+                               _p(shift), _p(next_weight), _p(out), _code(out.dtype) if out is not None else 0,
+                               _p(rows), n, H, float(eps_branch), float(eps_next), _stream()), lib)
+    return out
+
+
+def add_row(h: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """h[t, :] += v for every row of the float residual stream."""
+    _dev(h, v)
+    _f32(h, v)
+    if v.numel() != h.shape[1]:
+        raise KernelError(f"add_row: {v.numel()} values for rows of {h.shape[1]}")
+    lib = core()
+    _check(lib.lyp_add_row(_p(h), _p(v), h.shape[0], h.shape[1], _stream()), lib)
+    return h
+
+
+def short_conv(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor | None, q_start: torch.Tensor,
+               positions: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, B: int, residual: bool = True):
+    """out = (x +) the causal filter of x over time, channel by channel, request by request:
+    w float [C, taps]; ``state`` [slots, taps - 1, C] of x's type holds every request's last inputs
+    from earlier steps (not read for a request at position 0) and is brought up to date."""
+    _dev(x, w, state, q_start, positions, slots, out)
+    _f32(w)
+    T, C = x.shape
+    taps = w.shape[1]
+    if tuple(w.shape) != (C, taps) or out.shape != x.shape or out.dtype != x.dtype or out.data_ptr() == x.data_ptr():
+        raise KernelError(f"short_conv: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} {out.dtype}")
+    if taps > 1 and (state is None or state.dtype != x.dtype or tuple(state.shape[1:]) != (taps - 1, C)):
+        raise KernelError(f"short_conv: state {None if state is None else tuple(state.shape)} for {taps} taps of {C}")
+    if q_start.numel() != B + 1 or slots.numel() != B or positions.numel() != T:
+        raise KernelError("short_conv: the step's tables do not fit its rows and requests")
+    lib = core()
+    _check(lib.lyp_short_conv(_p(x), _p(w), _p(state), _p(q_start), _p(positions), _p(slots), _p(out), _code(x.dtype),
+                              T, B, C, taps, int(residual), _stream()), lib)
+    return out
+
+
+ACTIVATIONS = {"xielu": 0, "gelu_tanh": 1}
+
+
+def activation(x: torch.Tensor, kind: str, params: torch.Tensor | None = None,
+               out: torch.Tensor | None = None) -> torch.Tensor:
+    """Elementwise activation in 32-bit: "xielu" (params: its two learned numbers, float) or
+    "gelu_tanh".  In place unless ``out`` is given."""
+    out = x if out is None else out
+    _dev(x, params, out)
+    _f32(params)
+    if kind not in ACTIVATIONS or out.shape != x.shape or out.dtype != x.dtype or (kind == "xielu" and (
+            params is None or params.numel() != 2)):
+        raise KernelError(f"activation {kind!r} on {tuple(x.shape)} {x.dtype}")
+    lib = core()
+    _check(lib.lyp_activation(_p(x), _p(out), _code(x.dtype), x.numel(), ACTIVATIONS[kind], _p(params), _stream()), lib)
+    return out
+
+
+def mingru_scan(pre: torch.Tensor, bz: torch.Tensor, bx: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor,
+                positions: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, B: int) -> torch.Tensor:
+    """The minGRU recurrence over the step's rows, request by request: pre float [T, 3 W] holds the
+    update-gate, candidate and output-gate projections side by side; state float [slots, W]."""
+    _dev(pre, bz, bx, state, q_start, positions, slots, out)
+    _f32(pre, bz, bx, state)
+    T, W = out.shape
+    if tuple(pre.shape) != (T, 3 * W) or bz.numel() != W or bx.numel() != W or state.shape[1] != W or \
+            q_start.numel() != B + 1 or slots.numel() != B or positions.numel() != T:
+        raise KernelError(f"mingru_scan: pre {tuple(pre.shape)}, out {tuple(out.shape)}, state {tuple(state.shape)}")
+    lib = core()
+    _check(lib.lyp_mingru_scan(_p(pre), _p(bz), _p(bx), _p(state), _p(q_start), _p(positions), _p(slots), _p(out),
+                               _code(out.dtype), B, W, _stream()), lib)
+    return out
+
+
+def latent_prep(d: torch.Tensor, wq: torch.Tensor, wkv: torch.Tensor, positions: torch.Tensor,
+                table: torch.Tensor | None, slot_map: torch.Tensor, cq: torch.Tensor, pages: torch.Tensor, *,
+                q_rank: int, kv_rank: int, rot_dim: int, eps: float) -> None:
+    """From the down-projections of a step's rows (d [T, q_rank + kv_rank + rot_dim]): the normed
+    query latent into cq, and the normed key/value latent with the position-rotated shared key part
+    into each token's page slot (pages [pages, page size, kv_rank + rot_dim])."""
+    _dev(d, wq, wkv, positions, table, slot_map, cq, pages)
+    _f32(wq, wkv, table)
+    T = d.shape[0]
+    dims = 0 if table is None else table.shape[1]
+    if d.shape[1] != q_rank + kv_rank + rot_dim or tuple(cq.shape) != (T, q_rank) or cq.dtype != d.dtype or \
+            pages.dtype != d.dtype or pages.dim() != 3 or pages.shape[2] != kv_rank + rot_dim or \
+            wq.numel() != q_rank or wkv.numel() != kv_rank or positions.numel() != T or slot_map.numel() != T:
+        raise KernelError(f"latent_prep: d {tuple(d.shape)}, cq {tuple(cq.shape)}, pages {tuple(pages.shape)}")
+    lib = core()
+    _check(lib.lyp_latent_prep(_p(d), d.stride(0), _p(wq), _p(wkv), _p(positions), _p(table), dims, _p(slot_map),
+                               _p(cq), _p(pages), _code(d.dtype), T, q_rank, kv_rank, rot_dim, float(eps),
+                               _stream()), lib)
+
+
+def latent_query_rotate(q: torch.Tensor, positions: torch.Tensor, table: torch.Tensor | None, qa: torch.Tensor, *,
+                        num_heads: int, dim: int, rot_dim: int, kv_rank: int) -> None:
+    """The rotated part of every query head (q [T, H (dim + rot_dim)], the last rot_dim of each head),
+    turned by the token's position, into qa[:, head, kv_rank:] (qa [T, H, kv_rank + rot_dim])."""
+    _dev(q, positions, table, qa)
+    _f32(table)
+    T = q.shape[0]
+    dims = 0 if table is None else table.shape[1]
+    if q.shape[1] != num_heads * (dim + rot_dim) or tuple(qa.shape) != (T, num_heads, kv_rank + rot_dim) or \
+            qa.dtype != q.dtype or positions.numel() != T:
+        raise KernelError(f"latent_query_rotate: q {tuple(q.shape)}, qa {tuple(qa.shape)}")
+    lib = core()
+    _check(lib.lyp_latent_query_rotate(_p(q), _p(positions), _p(table), dims, _p(qa), _code(q.dtype), T, num_heads,
+                                       dim, rot_dim, kv_rank, _stream()), lib)
+
+
+def latent_attn_rows(qa: torch.Tensor, pages: torch.Tensor, block_tables: torch.Tensor, q_start: torch.Tensor,
+                     positions: torch.Tensor, ctx_len: torch.Tensor, sink: torch.Tensor, scale: float,
+                     out: torch.Tensor, *, kv_rank: int, rot_dim: int) -> torch.Tensor:
+    """Causal attention of every row over its request's latents in the pages, all heads sharing one
+    key per token (the page row) whose first kv_rank values are also the value; the softmax's
+    denominator holds exp(sink[head]) as well.  Any sizes; a workgroup per (row, head)."""
+    _dev(qa, pages, block_tables, q_start, positions, ctx_len, sink, out)
+    _f32(sink)
+    T, H, Dk = qa.shape
+    B = ctx_len.numel()
+    if Dk != kv_rank + rot_dim or pages.dim() != 3 or pages.shape[2] != Dk or pages.dtype != qa.dtype or \
+            tuple(out.shape) != (T, H, kv_rank) or out.dtype != qa.dtype or sink.numel() != H or \
+            block_tables.dtype != torch.int32 or block_tables.dim() != 2 or block_tables.shape[0] != B or \
+            q_start.numel() != B + 1 or positions.numel() != T:
+        raise KernelError(f"latent_attn_rows: qa {tuple(qa.shape)}, pages {tuple(pages.shape)}, out {tuple(out.shape)}")
+    lib = core()
+    _check(lib.lyp_latent_attn_rows(_p(qa), _p(pages), _p(block_tables), block_tables.shape[1], pages.shape[1],
+                                    _p(q_start), _p(positions), _p(ctx_len), B, _p(sink), float(scale), _p(out),
+                                    _code(qa.dtype), T, H, kv_rank, rot_dim, _stream()), lib)
     return out
 
 

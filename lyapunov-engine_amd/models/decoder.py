@@ -12,12 +12,12 @@ embedding matrix itself, not a copy (models/weight_loader.py:106-109 copies).
 from __future__ import annotations
 
 import fnmatch
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Iterator, Optional
 
 import torch
 
-from ..config.registry import BLOCKS, EMBEDDINGS, HEADS, NORMS
+from ..config.registry import BLOCKS, EMBEDDINGS, HEADS, NORMS, STREAM_SHIFTS
 from ..config.specs import LayerCall, ModelSpec
 from ..kernels import ops
 from ..parts.base import (LayerCache, Logits, PagedSpec, Part, PositionEncoding, StateSpec, StepContext, WeightSource,
@@ -33,7 +33,8 @@ class CacheGroupLayout:
 @dataclass(frozen=True)
 class CacheLayout:
     groups: tuple           # of CacheGroupLayout
-    states: dict            # cache id -> StateSpec
+    states: dict            # cache id -> StateSpec: the mixers'
+    part_states: dict = field(default_factory=dict)   # (cache id, name) -> StateSpec: other parts' (Block.state_specs)
 
     def group_of(self, cache_id: int) -> Optional[int]:
         for g, layout in enumerate(self.groups):
@@ -51,10 +52,14 @@ class DecoderModel(Part):
         self.head = HEADS.build(spec.head, vocab_size=spec.vocab_size, hidden_size=spec.hidden_size)
         if spec.tie_word_embeddings:
             self.head.tie(self.embedding)
+        self.stream_shift = STREAM_SHIFTS.build(spec.stream_shift, hidden_size=spec.hidden_size) \
+            if spec.stream_shift is not None else None
         self.schedule: tuple = tuple(spec.schedule)
         for call in self.schedule:
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"the running order names layer {call.layer}; there are {len(self.layers)}")
+            if call.shift is not None and self.stream_shift is None:
+                raise ValueError("a call of the running order adds a stream shift, and the model has none")
         self.device: Optional[torch.device] = None
         self.dtype: Optional[torch.dtype] = None
         self.max_positions = spec.max_position      # positions a step may reach; ``materialize`` may lower it
@@ -79,6 +84,8 @@ class DecoderModel(Part):
                 yield from walk(prefix + piece, child)
 
         yield from walk(self.spec.embed_prefix, self.embedding)
+        if self.stream_shift is not None:
+            yield from walk(self.spec.stream_shift_prefix, self.stream_shift)
         for i, layer in enumerate(self.layers):
             yield from walk(self.spec.layer_prefix.format(i=i), layer)
         yield from walk(self.spec.final_norm_prefix, self.final_norm)
@@ -115,9 +122,14 @@ class DecoderModel(Part):
     def _plan_cache(self) -> CacheLayout:
         by_cache: dict = {}
         states: dict = {}
+        part_states: dict = {}
         for call in self.schedule:
             mixer = self.layers[call.layer].mixer
             kv, st = mixer.cache_spec(), mixer.state_spec()
+            further = getattr(self.layers[call.layer], "state_specs", None)
+            for name, spec in (further() if further is not None else {}).items():
+                if part_states.setdefault((call.cache, name), spec) != spec:
+                    raise ValueError(f"state {name!r} of buffer {call.cache} is used with two shapes")
             if kv is not None:
                 if call.cache in by_cache and by_cache[call.cache] != kv:
                     raise ValueError(f"cache buffer {call.cache} is used with two shapes: {by_cache[call.cache]} and {kv}")
@@ -136,7 +148,7 @@ class DecoderModel(Part):
             if kv is not None and kv not in order:
                 order.append(kv)
         groups = tuple(CacheGroupLayout(kv, tuple(sorted(c for c, s in by_cache.items() if s == kv))) for kv in order)
-        return CacheLayout(groups, states)
+        return CacheLayout(groups, states, part_states)
 
     def cache_layout(self) -> CacheLayout:
         return self._layout
@@ -153,6 +165,8 @@ class DecoderModel(Part):
                 if isinstance(part, PositionEncoding):
                     part.limit_positions(self.max_positions)
         self.embedding.materialize(self.device, dtype)
+        if self.stream_shift is not None:
+            self.stream_shift.materialize(self.device, dtype)
         for layer in self.layers:
             layer.materialize(self.device, dtype)
         self.final_norm.materialize(self.device, dtype)
@@ -167,11 +181,15 @@ class DecoderModel(Part):
         h = self.embedding.forward(ctx, ctx.token_ids)
         delta = None
         for call, cache in zip(self.schedule, caches):
+            if call.shift is not None:
+                delta = ops.shifted(h, delta, self.stream_shift.row(call.shift))
             h, delta = self.layers[call.layer].forward(ctx, h, delta, cache)
         if ctx.R == 0:
             return None
         if isinstance(delta, ops.PendingLinear) and not getattr(self.final_norm, "can_defer", False):
             delta = delta.run()
+        if isinstance(delta, ops.JoiningBranch) and not getattr(self.final_norm, "joins_branches", False):
+            delta = delta.join(h)
         x = self.final_norm.forward(ctx, h, delta, rows=ctx.logit_rows)
         out = self.head.forward(ctx, x)
         return out if isinstance(out, Logits) else Logits(out)

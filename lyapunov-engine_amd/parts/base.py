@@ -126,7 +126,7 @@ class StateSpec:
     that carry a summary instead of keys."""
 
     shape: tuple
-    dtype: torch.dtype = torch.float32
+    dtype: Optional[torch.dtype] = torch.float32    # None: the engine's activation type
 
 
 @dataclass
@@ -146,8 +146,9 @@ class LayerCache:
 
     group: Optional[GroupView] = None
     pages: dict = field(default_factory=dict)   # PageTensor.name -> [pages, *PageTensor.page_shape(page size)]
-    state: Optional[torch.Tensor] = None  # [slots, *StateSpec.shape]
+    state: Optional[torch.Tensor] = None  # [slots, *StateSpec.shape]: the mixer's
     writes: bool = True                   # false: read what another call stored
+    states: dict = field(default_factory=dict)  # the block's further states by name (Block.state_specs)
 
     @property
     def k(self) -> Optional[torch.Tensor]:
@@ -343,6 +344,25 @@ class Mixer(Part):
         raise NotImplementedError
 
 
+class InputFilter(Part):
+    """Works over time on what a branch reads, channel by channel, within each
+    request; what it has to remember between steps lives in a state slot."""
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, state: Optional[torch.Tensor]) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class StreamShift(Part):
+    """A table of vectors; ``row(i)`` is the float vector [hidden] that the
+    decoder adds to every row of the residual stream before a call that names i."""
+
+    def row(self, i: int) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class FeedForward(Part):
     takes_pending_norm = False   # as for Mixer
 
@@ -356,6 +376,12 @@ class Block(Part):
 
     mixer: Mixer
 
+    def state_specs(self) -> dict:
+        """State per live request that parts of the arrangement other than the
+        mixer keep (an input filter's last inputs, ...): name -> StateSpec; the
+        tensors reach ``forward`` as ``cache.states[name]``."""
+        return {}
+
     def forward(self, ctx: StepContext, h: torch.Tensor, delta: Optional[torch.Tensor],
                 cache: LayerCache) -> tuple:
         """-> (h, delta): the residual stream and the output not yet added to it."""
@@ -365,5 +391,5 @@ class Block(Part):
 __all__ = [
     "WeightSource", "WeightSpec", "Part", "PagedSpec", "PageTensor", "SLOT", "StateSpec", "GroupView", "LayerCache", "StepContext",
     "StepBatch", "StepPlan", "StepPlanner", "FixedStep",
-    "Norm", "PositionEncoding", "Mixer", "FeedForward", "Block", "Logits", "Any",
+    "Norm", "PositionEncoding", "Mixer", "FeedForward", "InputFilter", "StreamShift", "Block", "Logits", "Any",
 ]

@@ -8,7 +8,7 @@ added.
 """
 from __future__ import annotations
 
-from ..config.registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+from ..config.registry import BLOCKS, FEED_FORWARDS, FILTERS, MIXERS, NORMS
 from ..config.specs import LayerSpec
 from ..kernels import ops
 from .base import Block, LayerCache, StepContext
@@ -35,10 +35,64 @@ class PreNormBlock(Block):
         return h, self.ffn.forward(ctx, x)
 
 
+@BLOCKS.register("sandwich")
+class SandwichBlock(Block):
+    """A norm in front of and behind each branch, a multiplier on what joins,
+    and optionally a filter over time on what the mixer reads:
+
+        h += mult * norm1_out(mixer(filter(norm1(h))));  h += mult * norm2_out(ffn(norm2(h)))
+
+    The feed-forward branch may be absent (``LayerSpec.ffn`` None).  The further
+    parts come from ``LayerSpec.extra``: "norm1_out", "norm2_out" (norms) and
+    "filter" (an input filter); ``LayerSpec.params["mult"]`` is the multiplier.
+    A branch's join is carried out by the norm that follows it, in one kernel
+    (ops.JoiningBranch); the block returns its last branch still to be joined."""
+
+    def __init__(self, spec: LayerSpec):
+        self.names = dict(spec.names)
+        self.mult = float(spec.params.get("mult", 1.0))
+        self.norm1 = NORMS.build(spec.norm1)
+        self.mixer = MIXERS.build(spec.mixer)
+        self.norm1_out = NORMS.build(spec.extra["norm1_out"])
+        self.filter = FILTERS.build(spec.extra["filter"]) if "filter" in spec.extra else None
+        self.ffn = FEED_FORWARDS.build(spec.ffn) if spec.ffn is not None else None
+        self.norm2 = NORMS.build(spec.norm2) if self.ffn is not None else None
+        self.norm2_out = NORMS.build(spec.extra["norm2_out"]) if self.ffn is not None else None
+        unknown = set(spec.extra) - {"norm1_out", "norm2_out", "filter"}
+        if unknown:
+            raise ValueError(f"the sandwich arrangement has no parts {sorted(unknown)}")
+
+    def children(self):
+        n = self.names
+        out = {n["norm1"]: self.norm1, n["mixer"]: self.mixer, n["norm1_out"]: self.norm1_out}
+        if self.filter is not None:
+            out[n["filter"]] = self.filter
+        if self.ffn is not None:
+            out.update({n["norm2"]: self.norm2, n["ffn"]: self.ffn, n["norm2_out"]: self.norm2_out})
+        return out
+
+    def state_specs(self):
+        st = self.filter.state_spec() if self.filter is not None else None
+        return {"filter": st} if st is not None else {}
+
+    def forward(self, ctx: StepContext, h, delta, cache: LayerCache):
+        x = normed(self.norm1, None, ctx, h, delta)
+        if self.filter is not None:
+            x = self.filter.forward(ctx, x, cache.states.get("filter"))
+        branch = self.norm1_out.branch(self.mixer.forward(ctx, x, cache), self.mult)
+        if self.ffn is None:
+            return h, branch
+        x = self.norm2.forward(ctx, h, branch)
+        return h, self.norm2_out.branch(self.ffn.forward(ctx, x), self.mult)
+
+
 def normed(norm, consumer, ctx: StepContext, h, delta):
     """h += delta; the normed rows for ``consumer``.  A norm that can and a
     consumer that takes it may pass the rows on unevaluated (ops.PendingNorm);
-    a norm that does not know of pending products gets the product itself."""
+    a norm that does not know of pending products gets the product itself, and
+    one that does not know of joining branches finds the branch joined."""
+    if isinstance(delta, ops.JoiningBranch) and not getattr(norm, "joins_branches", False):
+        delta = delta.join(h)
     if getattr(norm, "can_defer", False):
         return norm.forward(ctx, h, delta, lazy=getattr(consumer, "takes_pending_norm", False))
     if isinstance(delta, ops.PendingLinear):

@@ -14,29 +14,32 @@ from typing import Optional
 
 import torch
 
-from ..config.registry import EMBEDDINGS, HEADS
+from ..config.registry import EMBEDDINGS, HEADS, STREAM_SHIFTS
 from ..kernels import ops
-from .base import Embedding, Head, Logits, StepContext, WeightSource, WeightSpec
+from .base import Embedding, Head, Logits, StepContext, StreamShift, WeightSource, WeightSpec
 
 
 @EMBEDDINGS.register("lookup")
 class TokenEmbedding(Embedding):
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, tensor: str = "weight"):
+        """``scale`` multiplies every row that is looked up; ``tensor`` is what the matrix is called
+        after the part's prefix."""
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
+        self.scale, self.tensor = float(scale), tensor
         self.weight: Optional[torch.Tensor] = None
 
     def weight_specs(self):
-        return [WeightSpec("weight", (WeightSource("weight", (self.vocab_size, self.hidden_size)),))]
+        return [WeightSpec("weight", (WeightSource(self.tensor, (self.vocab_size, self.hidden_size)),))]
 
     def forward(self, ctx: StepContext, token_ids: torch.Tensor) -> torch.Tensor:
         h = torch.empty((token_ids.numel(), self.hidden_size), dtype=torch.float32, device=ctx.device)
-        return ops.embedding(token_ids, self.weight, h)
+        return ops.embedding(token_ids, self.weight, h, self.scale)
 
 
 @HEADS.register("linear")
 class LinearHead(Head):
-    def __init__(self, vocab_size: int, hidden_size: int):
-        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+    def __init__(self, vocab_size: int, hidden_size: int, tensor: str = "weight"):
+        self.vocab_size, self.hidden_size, self.tensor = vocab_size, hidden_size, tensor
         self.weight: Optional[torch.Tensor] = None
         self._tied_to: Optional[Embedding] = None
 
@@ -46,7 +49,7 @@ class LinearHead(Head):
     def weight_specs(self):
         if self._tied_to is not None:
             return []
-        return [WeightSpec("weight", (WeightSource("weight", (self.vocab_size, self.hidden_size)),))]
+        return [WeightSpec("weight", (WeightSource(self.tensor, (self.vocab_size, self.hidden_size)),))]
 
     def materialize(self, device, dtype):
         if self._tied_to is not None:
@@ -54,3 +57,25 @@ class LinearHead(Head):
 
     def forward(self, ctx: StepContext, x: torch.Tensor) -> Logits:
         return Logits(*ops.lm_head(x, self.weight))
+
+
+@STREAM_SHIFTS.register("table")
+class ShiftTable(StreamShift):
+    """``count`` learned vectors of the stream's width in one tensor [count, hidden]; a call of the
+    running order that names row i has it added to every row of the residual stream."""
+
+    def __init__(self, count: int, hidden_size: int, tensor: str = "weight"):
+        self.count, self.hidden_size, self.tensor = int(count), int(hidden_size), tensor
+        self.weight: Optional[torch.Tensor] = None
+        self.weight_f: Optional[torch.Tensor] = None
+
+    def weight_specs(self):
+        return [WeightSpec("weight", (WeightSource(self.tensor, (self.count, self.hidden_size)),))]
+
+    def materialize(self, device, dtype):
+        self.weight_f = self.weight.float().contiguous()
+
+    def row(self, i: int) -> torch.Tensor:
+        if not 0 <= i < self.count:
+            raise IndexError(f"stream shift {i} of {self.count}")
+        return self.weight_f[i]

@@ -1,0 +1,42 @@
+"""Filters over time on what a branch reads.
+
+"short_conv": a causal convolution with a few taps per channel, added to its
+input: out_t = x_t + sum_j w[:, j] * x_(t - taps + 1 + j), with zeros before the
+first token of a request.  The last taps - 1 inputs of every live request stay
+in a state slot, so that a prompt may be cut anywhere and a decoded token sees
+the tokens before it.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..config.registry import FILTERS
+from ..kernels import ops
+from .base import InputFilter, StateSpec, StepContext, WeightSource, WeightSpec
+
+
+@FILTERS.register("short_conv")
+class CausalShortConv(InputFilter):
+    def __init__(self, channels: int, taps: int, residual: bool = True, tensor: str = "weight"):
+        if taps < 1:
+            raise ValueError(f"a convolution needs at least one tap, not {taps}")
+        self.channels, self.taps, self.residual, self.tensor = int(channels), int(taps), bool(residual), tensor
+        self.weight: Optional[torch.Tensor] = None
+        self.weight_f: Optional[torch.Tensor] = None
+
+    def weight_specs(self):
+        return [WeightSpec("weight", (WeightSource(self.tensor, (self.channels, self.taps)),))]
+
+    def materialize(self, device, dtype):
+        self.weight_f = self.weight.float().contiguous()
+
+    def state_spec(self):
+        # the inputs are activations; they are kept as they were read
+        return StateSpec((self.taps - 1, self.channels), None) if self.taps > 1 else None
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, state: Optional[torch.Tensor]) -> torch.Tensor:
+        out = torch.empty_like(x)
+        return ops.short_conv(x, self.weight_f, state, ctx.q_start, ctx.positions, ctx.state_slots, out, ctx.B,
+                              residual=self.residual)

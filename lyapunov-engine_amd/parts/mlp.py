@@ -16,6 +16,43 @@ from ..kernels import ops
 from .base import FeedForward, StepContext, WeightSource, WeightSpec
 
 
+@FEED_FORWARDS.register("dense")
+class DenseFeedForward(FeedForward):
+    """down(act(up(x))), no gate and no biases.  ``activation``: "xielu", with its two learned
+    numbers p, q in one tensor (z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q)) (e^z - 1 - z)
+    + z/2), or "gelu_tanh"."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "xielu",
+                 names: Optional[dict] = None):
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {sorted(ops.ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size, self.activation = int(hidden_size), int(intermediate_size), activation
+        n = dict(up="up", down="down", act="act")
+        n.update(names or {})
+        self.names = n
+        self.up_proj: Optional[torch.Tensor] = None
+        self.down_proj: Optional[torch.Tensor] = None
+        self.act_params: Optional[torch.Tensor] = None
+        self.act_params_f: Optional[torch.Tensor] = None
+
+    def weight_specs(self):
+        n = self.names
+        specs = [WeightSpec("up_proj", (WeightSource(n["up"], (self.intermediate_size, self.hidden_size)),)),
+                 WeightSpec("down_proj", (WeightSource(n["down"], (self.hidden_size, self.intermediate_size)),))]
+        if self.activation == "xielu":
+            specs.append(WeightSpec("act_params", (WeightSource(n["act"], (2,)),)))
+        return specs
+
+    def materialize(self, device, dtype):
+        if self.act_params is not None:
+            self.act_params_f = self.act_params.float().contiguous()
+
+    def forward(self, ctx: StepContext, x):
+        up = ops.linear(x, self.up_proj, out_dtype=ctx.dtype)
+        ops.activation(up, self.activation, self.act_params_f)
+        return ops.linear(up, self.down_proj, out_dtype=ctx.dtype)
+
+
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
     def __init__(self, hidden_size: int, intermediate_size: int):

@@ -19,19 +19,46 @@ from .base import Norm, StepContext, WeightSource, WeightSpec
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, tensor: str = "weight"):
+        """``tensor``: what the weight is called after the part's prefix ("" where the prefix is
+        the tensor's whole name)."""
         self.size = size
         self.eps = float(eps)
+        self.tensor = tensor
         self.weight: Optional[torch.Tensor] = None
+        self._weight_f: Optional[torch.Tensor] = None
 
     def weight_specs(self):
-        return [WeightSpec("weight", (WeightSource("weight", (self.size,)),), init="ones")]
+        return [WeightSpec("weight", (WeightSource(self.tensor, (self.size,)),), init="ones")]
+
+    @property
+    def weight_f(self) -> torch.Tensor:
+        """The weights as float (made on first use; a norm's weights do not change)."""
+        if self._weight_f is None:
+            self._weight_f = self.weight.float().contiguous()
+        return self._weight_f
+
+    def branch(self, y, mult: float = 1.0) -> "ops.JoiningBranch":
+        """``y`` as a branch that joins the residual stream through this norm: mult * rmsnorm(y) * weight."""
+        if isinstance(y, ops.PendingLinear):
+            y = y.run()
+        if y.dim() == 3:
+            y = ops.sum_parts(y, torch.float32)
+        return ops.JoiningBranch(y, self.weight_f, self.eps, mult)
+
+    # A delta may be an ops.JoiningBranch: the sum and this norm are then one kernel.
+    joins_branches = True
 
     # With ``lazy`` the norm may add the delta and hand the rows on as an
     # ops.PendingNorm for the consumer's kernel to norm on its way in.
     can_defer = True
 
     def forward(self, ctx: StepContext, h, delta=None, rows=None, lazy=False):
+        if isinstance(delta, ops.JoiningBranch):
+            n = h.shape[0] if rows is None else rows.numel()
+            out = torch.empty((n, self.size), dtype=ctx.dtype, device=h.device)
+            return ops.branch_join(h, delta.y, delta.weight, delta.mult, delta.eps, shift=delta.shift,
+                                   next_weight=self.weight_f, eps_next=self.eps, out=out, rows=rows)
         if lazy and rows is None:
             pending, delta = ops.rmsnorm_pending(h, self.weight, self.eps, ctx.dtype, delta)
             if pending is not None:
