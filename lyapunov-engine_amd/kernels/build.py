@@ -39,12 +39,15 @@ CXX_FLAGS = ["-O2", "-std=c++20", "-fPIC", "-Wall", "-Wextra"]
 CORE_SOURCES = ["kernels/errors.hip", "kernels/elementwise.hip", "kernels/sequence.hip", "kernels/gemm.hip",
                 "kernels/sampler.hip"]
 ATTN_SOURCES = ["kernels/errors.hip", "kernels/attention.hip"]
+LATENT_SOURCES = ["kernels/errors.hip", "kernels/latent_attention.hip"]
 BLAS_SOURCES = ["kernels/errors.hip", "kernels/library_gemm.hip"]   # host code around the vendor's GEMM library
 RUNTIME_SOURCES = ["runtime/cache_manager.cpp", "runtime/scheduler.cpp", "runtime/c_api.cpp"]
 
 # Head sizes compiled ahead of time by build_all(); any other multiple of 16 up
 # to 256 is compiled when a model first asks for it.
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
+# (latent, rotated part) sizes of the latent attention library compiled ahead of time; others on first use.
+PREBUILT_LATENT_SIZES = ((64, 32), (96, 16), (64, 16), (256, 32))
 
 _lock = threading.Lock()
 
@@ -192,6 +195,15 @@ def attention_library(head_dim: int, force: bool = False) -> Path:
                          defines={"LYP_HEAD_DIM": str(head_dim)}, force=force)
 
 
+def latent_attention_library(kv_rank: int, rot_dim: int, force: bool = False) -> Path:
+    """The matrix-core attention over latents for one pair of sizes (compile-time constants there)."""
+    if kv_rank % 16 or rot_dim % 16 or not 16 <= kv_rank <= 512 or not 0 <= rot_dim <= 256:
+        raise ValueError(f"the latent attention kernels take latents of 16 to 512 values and rotated parts of up to "
+                         f"256, in multiples of 16, not {kv_rank} and {rot_dim}")
+    return build_library(f"lyp_latent_kv{kv_rank}_r{rot_dim}", LATENT_SOURCES, hip=True,
+                         defines={"LYP_LATENT_KV": str(kv_rank), "LYP_LATENT_RD": str(rot_dim)}, force=force)
+
+
 def blas_library(force: bool = False) -> Path:
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     return build_library("lyp_blas", BLAS_SOURCES, hip=True, force=force,
@@ -246,4 +258,6 @@ def build_all(force: bool = True) -> list[Path]:
     out = [runtime_library(force), core_library(force), blas_library(force)]
     for hd in PREBUILT_HEAD_DIMS:
         out.append(attention_library(hd, force))
+    for kv, rd in PREBUILT_LATENT_SIZES:
+        out.append(latent_attention_library(kv, rd, force))
     return out

@@ -998,6 +998,73 @@ def latent_attn_rows(qa: torch.Tensor, pages: torch.Tensor, block_tables: torch.
     return out
 
 
+_latent: dict = {}
+
+
+def latent_lib(kv_rank: int, rot_dim: int) -> ctypes.CDLL:
+    lib = _latent.get((kv_rank, rot_dim))
+    if lib is None:
+        lib = _load(build.latent_attention_library(kv_rank, rot_dim))
+        lib.lyp_last_error.restype = ctypes.c_char_p
+        if (lib.lyp_latent_kv_rank(), lib.lyp_latent_rot_dim()) != (kv_rank, rot_dim):
+            raise KernelError(f"latent attention library for sizes {kv_rank}, {rot_dim} reports others")
+        lib.lyp_latent_plan.argtypes = [c_int, c_int, c_int]
+        lib.lyp_latent_tile_keys.argtypes = [c_int]
+        lib.lyp_latent_attn.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                        c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                        c_void_p, c_void_p, c_void_p]
+        _latent[(kv_rank, rot_dim)] = lib
+    return lib
+
+
+def latent_attn_fits_matrix_cores(kv_rank: int, rot_dim: int) -> bool:
+    return kv_rank % 16 == 0 and rot_dim % 16 == 0 and 16 <= kv_rank <= 512 and rot_dim <= 256
+
+
+def latent_attn_launch(T: int, B: int, H: int, max_ctx: int, dtype: torch.dtype, kv_rank: int, rot_dim: int,
+                       n_parts: int | None = None) -> dict:
+    """The launch shape of ``latent_attn`` for a step of T rows of B requests with contexts of up
+    to max_ctx: row groups, partitions of the keys, keys per partition, and the floats of the
+    partitions' workspaces (host values only)."""
+    lib = latent_lib(kv_rank, rot_dim)
+    code = _code(dtype)
+    row_groups = -(-T * H // 64) + B
+    tile = lib.lyp_latent_tile_keys(code)
+    if n_parts is None:
+        n_parts = lib.lyp_latent_plan(row_groups, max_ctx, code)
+    part_keys = max(tile, -(-(-(-max_ctx // n_parts)) // tile) * tile)
+    n_parts = max(1, -(-max_ctx // part_keys))
+    n = T * H * n_parts if n_parts > 1 else 0
+    return dict(row_groups=row_groups, n_parts=n_parts, part_keys=part_keys, part_o=n * kv_rank, part_ml=n * 2)
+
+
+def latent_attn(qa: torch.Tensor, pages: torch.Tensor, block_tables: torch.Tensor, q_start: torch.Tensor,
+                positions: torch.Tensor, ctx_len: torch.Tensor, sink: torch.Tensor, scale: float, out: torch.Tensor,
+                launch: dict, part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None, *,
+                kv_rank: int, rot_dim: int) -> torch.Tensor:
+    """``latent_attn_rows`` on the matrix cores (sizes in multiples of 16), a prompt's rows and
+    single tokens alike; ``launch`` comes from ``latent_attn_launch`` for a bound on the step's
+    contexts that the caller guarantees (keys beyond n_parts * part_keys would be left out)."""
+    _dev(qa, pages, block_tables, q_start, positions, ctx_len, sink, out, part_o, part_ml)
+    _f32(sink, part_o, part_ml)
+    T, H, Dk = qa.shape
+    B = ctx_len.numel()
+    if Dk != kv_rank + rot_dim or pages.dim() != 3 or pages.shape[2] != Dk or pages.dtype != qa.dtype or \
+            tuple(out.shape) != (T, H, kv_rank) or out.dtype != qa.dtype or sink.numel() != H or \
+            block_tables.dtype != torch.int32 or block_tables.dim() != 2 or block_tables.shape[0] != B or \
+            q_start.numel() != B + 1 or positions.numel() != T or launch["row_groups"] < -(-T * H // 64) + B:
+        raise KernelError(f"latent_attn: qa {tuple(qa.shape)}, pages {tuple(pages.shape)}, out {tuple(out.shape)}")
+    if launch["n_parts"] > 1 and (part_o is None or part_ml is None or part_o.numel() < launch["part_o"]
+                                  or part_ml.numel() < launch["part_ml"]):
+        raise KernelError("latent_attn: the partitions' workspace is missing or too small")
+    lib = latent_lib(kv_rank, rot_dim)
+    _check(lib.lyp_latent_attn(_p(qa), _p(pages), _p(block_tables), block_tables.shape[1], pages.shape[1], _p(q_start),
+                               _p(positions), _p(ctx_len), B, _p(sink), float(scale), _p(out), _code(qa.dtype), T, H,
+                               launch["row_groups"], launch["n_parts"], launch["part_keys"], _p(part_o), _p(part_ml),
+                               _stream()), lib)
+    return out
+
+
 # ------------------------------------------------------------------- attention
 def attn_decode_plan(n_seqs: int, max_ctx: int, num_heads: int, num_kv_heads: int, head_dim: int) -> int:
     """Keys per workgroup (the partition size) for a decode launch of this size."""

@@ -27,7 +27,22 @@ import torch
 from ..config.registry import MIXERS, POSITION_ENCODINGS
 from ..config.specs import PartSpec
 from ..kernels import ops
-from .base import SLOT, LayerCache, Mixer, PagedSpec, PageTensor, StepContext, WeightSource, WeightSpec
+from .base import (SLOT, LayerCache, Mixer, PagedSpec, PageTensor, StepBatch, StepContext, StepPlanner, WeightSource,
+                   WeightSpec)
+
+
+class ContextBound(StepPlanner):
+    """The longest context of the step, as a host value (``meta["max_ctx"]``; in a recorded step
+    the step's bound): what a kernel that cuts the keys into partitions sizes its launch by."""
+
+    key = ("context_bound",)
+
+    def plan(self, batch: StepBatch) -> tuple:
+        bound = batch.fixed.max_context if batch.fixed is not None else int(batch.ctx_len.max())
+        return {}, dict(max_ctx=max(1, bound))
+
+
+_BOUND = ContextBound()
 
 
 @MIXERS.register("latent_attention")
@@ -50,6 +65,8 @@ class LatentAttention(Mixer):
         n = dict(dq="dq", q_norm="dq.norm", uq="uq", dkv="dkv", kv_norm="dkv.norm", uk="uk", uv="uv", sink="sink", o="o")
         n.update(names or {})
         self.names = n
+        # sizes in multiples of 16 take the matrix-core kernel, any others the row-by-row one
+        self.matrix_cores = ops.latent_attn_fits_matrix_cores(self.kv_rank, self.rot_dim)
         self.down_proj = self.q_norm = self.kv_norm = self.uq = self.uk = self.uv = self.sink = self.o_proj = None
         self.q_norm_f = self.kv_norm_f = self.sink_f = self.uk_t = self.uv_heads = None
 
@@ -82,6 +99,9 @@ class LatentAttention(Mixer):
         self.uk = None
         self.uv_heads = self.uv.view(H, self.vdim, self.kv_rank)
 
+    def step_planner(self):
+        return _BOUND
+
     def cache_spec(self):
         return PagedSpec((PageTensor("latent", (SLOT, self.kv_rank + self.rot_dim)),), 0)
 
@@ -104,9 +124,20 @@ class LatentAttention(Mixer):
             qa[:, :, :self.kv_rank].zero_()
         ops.latent_query_rotate(q, ctx.positions, table, qa, num_heads=H, dim=self.dim, rot_dim=self.rot_dim,
                                 kv_rank=self.kv_rank)
-        mixed = torch.empty((T, H, self.kv_rank), dtype=ctx.dtype, device=dev)
-        ops.latent_attn_rows(qa, pages, g.block_tables, ctx.q_start, ctx.positions, ctx.ctx_len, self.sink_f,
-                             self.scale, mixed, kv_rank=self.kv_rank, rot_dim=self.rot_dim)
+        # a recorded step may hold rows that belong to no request: nothing writes them
+        mixed = (torch.zeros if ctx.fixed is not None else torch.empty)((T, H, self.kv_rank), dtype=ctx.dtype, device=dev)
+        if self.matrix_cores:
+            launch = ops.latent_attn_launch(T, ctx.B, H, ctx.plans[ContextBound.key].meta["max_ctx"], ctx.dtype,
+                                            self.kv_rank, self.rot_dim)
+            part_o = part_ml = None
+            if launch["n_parts"] > 1:
+                part_o = ctx.scratch("latent_part_o", launch["part_o"])
+                part_ml = ctx.scratch("latent_part_ml", launch["part_ml"])
+            ops.latent_attn(qa, pages, g.block_tables, ctx.q_start, ctx.positions, ctx.ctx_len, self.sink_f,
+                            self.scale, mixed, launch, part_o, part_ml, kv_rank=self.kv_rank, rot_dim=self.rot_dim)
+        else:
+            ops.latent_attn_rows(qa, pages, g.block_tables, ctx.q_start, ctx.positions, ctx.ctx_len, self.sink_f,
+                                 self.scale, mixed, kv_rank=self.kv_rank, rot_dim=self.rot_dim)
         heads = torch.empty((T, H, self.vdim), dtype=ctx.dtype, device=dev)
         ops.gemm_nt_heads(mixed, self.uv_heads, heads)
         return ops.linear(heads.view(T, H * self.vdim), self.o_proj, out_dtype=ctx.dtype)

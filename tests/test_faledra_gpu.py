@@ -168,8 +168,17 @@ def latent_case(dtype, T_ctx, H, kv_rank, rot_dim, page_size, seed, n_new, use_m
     return keys, qa, sink
 
 
-def run_latent_attention(dtype, keys, qa, sink, scale, kv_rank, rot_dim, page_size, n_pages_extra=3, shuffle_seed=0):
+KERNELS = ["rows", "cores", "cores in 3 partitions"]
+
+
+def run_latent_attention(dtype, keys, qa, sink, scale, kv_rank, rot_dim, page_size, n_pages_extra=3, shuffle_seed=0,
+                         kernel="rows"):
+    """``kernel``: "rows" (any sizes, a workgroup per row and head) or "cores" (the matrix-core kernel;
+    sizes in multiples of 16), the latter also with the keys forced into partitions."""
     from lyapunov_engine_amd.kernels import ops
+
+    if kernel != "rows" and not ops.latent_attn_fits_matrix_cores(kv_rank, rot_dim):
+        pytest.skip("sizes that only the row-by-row kernel takes")
 
     T_ctx, Dk = keys.shape
     n_new, H = qa.shape[0], qa.shape[1]
@@ -183,8 +192,16 @@ def run_latent_attention(dtype, keys, qa, sink, scale, kv_rank, rot_dim, page_si
         pages[page_ids[j // page_size], j % page_size] = keys[j]
     to = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)
     out = torch.empty(n_new, H, kv_rank, dtype=tdt(dtype), device=DEV)
-    ops.latent_attn_rows(qa.to(DEV), pages.to(DEV), to([page_ids]), to([0, n_new]), to(np.arange(T_ctx - n_new, T_ctx)),
-                         to([T_ctx]), sink.to(DEV), scale, out, kv_rank=kv_rank, rot_dim=rot_dim)
+    args = (qa.to(DEV), pages.to(DEV), to([page_ids]), to([0, n_new]), to(np.arange(T_ctx - n_new, T_ctx)), to([T_ctx]),
+            sink.to(DEV), scale, out)
+    if kernel == "rows":
+        ops.latent_attn_rows(*args, kv_rank=kv_rank, rot_dim=rot_dim)
+        return out
+    launch = ops.latent_attn_launch(n_new, 1, H, T_ctx, tdt(dtype), kv_rank, rot_dim,
+                                    n_parts=3 if "partitions" in kernel else None)
+    part_o = torch.full((max(1, launch["part_o"]),), float("nan"), device=DEV)
+    part_ml = torch.full((max(1, launch["part_ml"]),), float("nan"), device=DEV)
+    ops.latent_attn(*args, launch, part_o, part_ml, kv_rank=kv_rank, rot_dim=rot_dim)
     return out
 
 
@@ -202,20 +219,23 @@ def plain_latent_attention(keys, qa, sink, scale, kv_rank):
     return out
 
 
+@pytest.mark.parametrize("kernel", KERNELS)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(37, 3, 40, 8, 4, 37), (300, 2, 24, 14, 16, 5), (130, 5, 64, 32, 16, 1),
-                                   (1000, 4, 96, 16, 16, 1), (513, 1, 48, 16, 16, 70)])
-def test_latent_attention_over_pages(dtype, shape):
+                                   (1000, 4, 96, 16, 16, 1), (513, 1, 48, 16, 16, 70), (700, 3, 32, 0, 16, 300),
+                                   (2100, 20, 16, 16, 64, 3)])
+def test_latent_attention_over_pages(dtype, shape, kernel):
     T_ctx, H, kv_rank, rot_dim, page_size, n_new = shape
     keys, qa, sink = latent_case(dtype, T_ctx, H, kv_rank, rot_dim, page_size, seed=T_ctx, n_new=n_new)
     scale = (kv_rank + rot_dim) ** -0.5
-    got = run_latent_attention(dtype, keys, qa, sink, scale, kv_rank, rot_dim, page_size)
+    got = run_latent_attention(dtype, keys, qa, sink, scale, kv_rank, rot_dim, page_size, kernel=kernel)
     close(got, plain_latent_attention(keys, qa, sink, scale, kv_rank), dtype, f"latent attention {shape}")
 
 
+@pytest.mark.parametrize("kernel", KERNELS)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("where", [0, 1, 15, 16, 17, 255, 256, 600, 898, 899])
-def test_latent_attention_finds_one_planted_key(dtype, where):
+@pytest.mark.parametrize("where", [0, 1, 15, 16, 17, 63, 64, 255, 256, 319, 320, 600, 898, 899])
+def test_latent_attention_finds_one_planted_key(dtype, where, kernel):
     """Among 900 keys one is made to carry the result (its score stands far above the rest): first
     tokens, page borders, far back, and the row's own position.  The sink is far below."""
     T_ctx, H, kv_rank, rot_dim, page_size = 900, 2, 32, 16, 16
@@ -223,25 +243,26 @@ def test_latent_attention_finds_one_planted_key(dtype, where):
     keys = (keys.float() * 0.1).to(tdt(dtype))
     qa = (keys[where].float() * 400.0)[None, None, :].repeat(1, H, 1).to(tdt(dtype))
     sink = torch.full((H,), -50.0)
-    got = run_latent_attention(dtype, keys, qa, sink, 1.0, kv_rank, rot_dim, page_size, shuffle_seed=where)
+    got = run_latent_attention(dtype, keys, qa, sink, 1.0, kv_rank, rot_dim, page_size, shuffle_seed=where, kernel=kernel)
     want = plain_latent_attention(keys, qa, sink, 1.0, kv_rank)
     close(got, want, dtype, f"planted key at {where}")
     assert torch.allclose(want[0, 0], keys[where, :kv_rank].double(), atol=0.05), "the planted key must carry the result"
 
 
+@pytest.mark.parametrize("kernel", KERNELS)
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_latent_attention_sink_takes_weight_and_the_future_is_not_seen(dtype):
+def test_latent_attention_sink_takes_weight_and_the_future_is_not_seen(dtype, kernel):
     T_ctx, H, kv_rank, rot_dim, page_size = 64, 3, 16, 16, 16
     keys, qa, sink = latent_case(dtype, T_ctx, H, kv_rank, rot_dim, page_size, seed=9, n_new=20)
     sink = torch.tensor([30.0, 0.0, -30.0])                                # head 0: nearly everything goes to the sink
-    got = run_latent_attention(dtype, keys, qa, sink, 0.2, kv_rank, rot_dim, page_size)
+    got = run_latent_attention(dtype, keys, qa, sink, 0.2, kv_rank, rot_dim, page_size, kernel=kernel)
     want = plain_latent_attention(keys, qa, sink, 0.2, kv_rank)
     close(got, want, dtype, "sinks")
     assert float(got[:, 0].abs().max()) < 1e-6 < float(got[:, 2].abs().max())
     # a key just after a row's position, made overwhelming, must not be seen by that row
     keys2 = keys.clone()
     keys2[50] = (qa[5, 1].float() * 50).to(tdt(dtype))                     # row 5 stands at position 49
-    got2 = run_latent_attention(dtype, keys2, qa, sink, 0.2, kv_rank, rot_dim, page_size)
+    got2 = run_latent_attention(dtype, keys2, qa, sink, 0.2, kv_rank, rot_dim, page_size, kernel=kernel)
     close(got2[:6], want[:6], dtype, "rows before the planted key")
     assert float((got2[6:].double().cpu() - want[6:]).abs().max()) > 0.1
 
