@@ -60,6 +60,108 @@ def build_engine(layers, dtype, num_blocks, max_num_seqs, block_size, budget, sh
     return engine, cfg
 
 
+# ------------------------------------------------------------ another design beside the Llama shape
+# Faledra models whose layers have the sizes of a real model's, each beside the Llama shape of equal
+# width, depth and feed-forward parameters (a dense feed-forward of 1.5 x the gated one's width has
+# the same three width x ff matrices' worth of weights): three latent-attention layers and one minGRU
+# layer in turn, a filter of three taps, the first four layers run twice.
+def faledra_shape(width, heads, ff, layers, vocab, q_rank, kv_rank):
+    def latent():
+        return dict(type="latent_attention", mlp=dict(kind="dense", ff=ff * 3 // 2),
+                    mixer=dict(heads=heads, dim=64, rot_dim=32, vdim=64, q_rank=q_rank, kv_rank=kv_rank,
+                               scale=96 ** -0.5, rot=dict(base=500000.0, dims=32)))
+
+    def gru():
+        return dict(type="mingru", mixer=dict(width=width), mlp=dict(kind="dense", ff=ff * 3 // 2))
+
+    return dict(architecture="Faledra", vocab=vocab, width=width, residual_mult=0.5, embedding=dict(scale=1.0),
+                norm=dict(eps=1e-5), canon=dict(taps=3), loop=dict(start=0, stop=4, times=2),
+                layers=[gru() if i % 4 == 3 else latent() for i in range(layers)])
+
+
+# name -> (Faledra configuration, the Llama shape beside it); the looped stretch makes layers + 4 layer runs
+DESIGN_SIZES = {
+    "small": (faledra_shape(1024, 16, 4096, 4, 32000, 384, 128),
+              dict(MODEL, vocab_size=32000, hidden_size=1024, intermediate_size=4096, num_hidden_layers=8,
+                   num_attention_heads=16, num_key_value_heads=4)),
+    "1b": (faledra_shape(2048, 32, 8192, 12, 128256, 768, 256), dict(MODEL, num_hidden_layers=16)),
+    "wide": (faledra_shape(4096, 32, 14336, 4, 128256, 1536, 512),
+             dict(SHAPES["8b"], num_hidden_layers=8, head_dim=128)),
+}
+
+
+def build_engine_from_config(raw, dtype, num_blocks, max_num_seqs, block_size, budget, max_model_len):
+    """An engine for any registered architecture's config.json contents, with random weights."""
+    import torch
+
+    from lyapunov_engine_amd.config import EngineConfig
+    from lyapunov_engine_amd.config.registry import architecture_of
+    from lyapunov_engine_amd.engine.core import EngineCore
+    from lyapunov_engine_amd.engine.llm_engine import LLMEngine
+    from lyapunov_engine_amd.models import build_model
+    from lyapunov_engine_amd.weights import DictSource, load_weights, random_tensors
+
+    arch = architecture_of(raw)
+    cfg = arch.config_class.from_dict(raw)
+    model = build_model(arch.to_spec(cfg))
+    tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tensors = dict(random_tensors(model, 4, tdtype, device="cuda:0"))
+    reach = min(num_blocks * block_size, max_model_len)
+    load_weights(model, DictSource(tensors), tdtype, "cuda:0", max_positions=reach)
+    del tensors
+    core = EngineCore(model, cfg, dtype=tdtype, device="cuda:0", num_blocks=num_blocks, block_size=block_size,
+                      num_state_slots=max_num_seqs)
+    engine = LLMEngine(core, EngineConfig(dtype=tdtype, num_blocks=num_blocks, block_size=block_size,
+                                          max_num_seqs=max_num_seqs, max_num_batched_tokens=budget,
+                                          max_model_len=max_model_len))
+    return engine, cfg
+
+
+class _Vocab:
+    """What the measuring functions read of a configuration."""
+
+    def __init__(self, engine):
+        self.vocab_size = engine.core.model.spec.vocab_size
+
+
+def run_design(args):
+    """Prefill and decode speed of the Faledra sizes, each beside the Llama shape of equal size."""
+    import torch
+
+    context, block_size, out = 2304, 16, {}
+    for size in (args.size.split(",") if args.size else sorted(DESIGN_SIZES)):
+        faledra, llama = DESIGN_SIZES[size]
+        out[size] = {}
+        for name, raw in (("faledra", faledra), ("llama", llama)):
+            engine, _ = build_engine_from_config(raw, args.dtype, 8 * (context // block_size + 1) + 64 + 2048 // block_size,
+                                                 8, block_size, budget=8192, max_model_len=context)
+            cfg = _Vocab(engine)
+            params = sum(t.numel() for part, ws in engine.core.model.weight_table() for t in [getattr(part, ws.attr)]
+                         if t is not None)
+            res = {"parameters_m": round(params / 1e6, 1)}
+            for tokens in (512, 2048):
+                s = measure_prefill(engine, cfg, tokens)
+                res[f"prefill_{tokens}_tok_s"] = round(tokens / s, 1)
+            for b in (1, 8):
+                s, _ = measure_decode(engine, cfg, b, context, min(args.steps, 64), min(args.warmup, 8), seed=30 + b)
+                res[f"decode_b{b}_ctx2048_tok_s"] = round(b / s, 1)
+                res[f"decode_b{b}_ms"] = round(s * 1e3, 4)
+            out[size][name] = res
+            del engine
+            torch.cuda.empty_cache()
+    first = out[sorted(out)[0]]
+    print(json.dumps({
+        "metric": "Faledra beside the Llama shape of equal size: prefill and decode tok/s", "unit": "tok/s",
+        "value": first["faledra"]["decode_b8_ctx2048_tok_s"], "n_gpus": 1, "steps": min(args.steps, 64),
+        "warmup": min(args.warmup, 8), "ms_per_step": first["faledra"]["decode_b8_ms"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic (random weights seed 4, random token ids)",
+        "config": {"model": "faledra", "sizes": sorted(out), "context_len": context, "kv_block_size": block_size,
+                   "parallelism": "single-gpu", "graphs": True},
+        "sizes": out}))
+    return 0
+
+
 def weight_bytes(cfg, esz):
     h, i = cfg.hidden_size, cfg.intermediate_size
     q, kv = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
@@ -269,10 +371,16 @@ def main():
                     help="mixed: the continuous batch of BASELINE.json configs[3] instead of the headline")
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode and the prefill")
     ap.add_argument("--skip-check", action="store_true", help="no comparison of bfloat16 logits with a 32-bit run")
+    ap.add_argument("--design", default="llama", choices=["llama", "faledra"],
+                    help="faledra: that design's prefill and decode speed at a few sizes, each beside the Llama "
+                         "shape of equal size, instead of the headline")
+    ap.add_argument("--size", default="", help="with --design faledra: which sizes, with commas (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.design == "faledra":
+        return run_design(args)
 
     import torch
 
