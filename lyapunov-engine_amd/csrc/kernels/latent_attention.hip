@@ -214,23 +214,27 @@ __global__ __launch_bounds__(64) void latent_combine_kernel(const float* __restr
                                                             const float* __restrict__ part_ml,
                                                             const float* __restrict__ sink, T* __restrict__ out,
                                                             int H, int n_parts) {
+  __shared__ float weight[256];   // at most 256 partitions (lyp_latent_attn checks)
   const size_t row = blockIdx.x;
   const int head = static_cast<int>(row % H);
   const float sk = sink[head];
+  // a lane a partition: maxima, weights and the denominator (partitions added in lane order)
   float mx = sk;
-  for (int p = 0; p < n_parts; ++p) mx = fmaxf(mx, part_ml[(row * n_parts + p) * 2]);
-  float denom = expf(sk - mx);
-  for (int p = 0; p < n_parts; ++p) {
+  for (int p = threadIdx.x; p < n_parts; p += kWave) mx = fmaxf(mx, part_ml[(row * n_parts + p) * 2]);
+  mx = wave_max(mx);
+  float part = 0.f;
+  for (int p = threadIdx.x; p < n_parts; p += kWave) {
     const float mp = part_ml[(row * n_parts + p) * 2];
-    if (mp > LYP_NEG_INF) denom += part_ml[(row * n_parts + p) * 2 + 1] * expf(mp - mx);
+    const float w = mp > LYP_NEG_INF ? expf(mp - mx) : 0.f;
+    weight[p] = w;
+    part += part_ml[(row * n_parts + p) * 2 + 1] * w;
   }
+  const float denom = wave_sum(part) + expf(sk - mx);
+  __syncthreads();
   const float inv = 1.0f / denom;
   for (int d = threadIdx.x; d < KV; d += kWave) {
     float acc = 0.f;
-    for (int p = 0; p < n_parts; ++p) {
-      const float mp = part_ml[(row * n_parts + p) * 2];
-      if (mp > LYP_NEG_INF) acc += part_o[(row * n_parts + p) * KV + d] * expf(mp - mx);
-    }
+    for (int p = 0; p < n_parts; ++p) acc += part_o[(row * n_parts + p) * KV + d] * weight[p];
     out[row * KV + d] = from_f32<T>(acc * inv);
   }
 }
@@ -253,9 +257,9 @@ int lyp_latent_tile_keys(int dtype) { return dtype == kF32 ? Tile<float>::kKeys 
 int lyp_latent_plan(int row_groups, int max_ctx, int dtype) {
   const int tile = lyp_latent_tile_keys(dtype);
   const int want = 2 * compute_units();
-  if (row_groups >= want || max_ctx <= 4 * tile) return 1;
+  if (row_groups >= want || max_ctx <= tile) return 1;
   int parts = (want + row_groups - 1) / row_groups;
-  parts = std::min(parts, (max_ctx + 4 * tile - 1) / (4 * tile));   // partitions of at least four tiles
+  parts = std::min(parts, (max_ctx + tile - 1) / tile);   // partitions of at least one tile
   return std::max(1, std::min(parts, 256));
 }
 
@@ -268,7 +272,7 @@ int lyp_latent_attn(const void* qa, const void* pages, const int32_t* block_tabl
                     int n_parts, int part_keys, float* part_o, float* part_ml, hipStream_t stream) {
   LYP_REQUIRE(n_rows >= 0 && B > 0 && H > 0 && page_size > 0 && table_width > 0 && row_groups > 0,
               "latent_attn: bad sizes rows=%d B=%d H=%d page=%d", n_rows, B, H, page_size);
-  LYP_REQUIRE(n_parts >= 1 && n_parts <= 65535 && part_keys > 0, "latent_attn: %d partitions of %d keys", n_parts,
+  LYP_REQUIRE(n_parts >= 1 && n_parts <= 256 && part_keys > 0, "latent_attn: %d partitions of %d keys", n_parts,
               part_keys);
   LYP_REQUIRE(part_keys % lyp_latent_tile_keys(dtype) == 0 || n_parts == 1,
               "latent_attn: partitions of %d keys are no multiple of the tile", part_keys);

@@ -89,13 +89,16 @@ def core() -> ctypes.CDLL:
         lib.lyp_gemm_nt_batched.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                             c_int, c_int, c_int, c_longlong, c_longlong, c_longlong, c_void_p]
         lib.lyp_branch_join.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
-                                        c_int, c_void_p, c_int, c_int, c_float, c_float, c_void_p]
+                                        c_int, c_void_p, c_int, c_int, c_float, c_float, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_int, c_void_p]
         lib.lyp_add_row.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p]
         lib.lyp_short_conv.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                        c_int, c_int, c_int, c_int, c_int, c_void_p]
         lib.lyp_activation.argtypes = [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p, c_void_p]
         lib.lyp_mingru_scan.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int, c_int, c_int, c_void_p]
+        lib.lyp_mingru_scan_chunks.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                               c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_longlong, c_void_p]
         lib.lyp_latent_prep.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]
         lib.lyp_latent_query_rotate.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
@@ -849,13 +852,28 @@ def _f32(*ts) -> None:
 
 def branch_join(h: torch.Tensor, y: torch.Tensor | None, branch_weight: torch.Tensor | None, mult: float,
                 eps_branch: float, *, shift: torch.Tensor | None = None, next_weight: torch.Tensor | None = None,
-                eps_next: float = 0.0, out: torch.Tensor | None = None, rows: torch.Tensor | None = None):
+                eps_next: float = 0.0, out: torch.Tensor | None = None, rows: torch.Tensor | None = None,
+                conv: tuple | None = None):
     """h += mult * rmsnorm(y) * branch_weight (+ shift, a vector added to every row), in 32-bit on the
     residual stream; with ``next_weight`` the sum's RMS norm times that weight goes to ``out``
     (activations).  ``rows`` picks the rows to join and norm into ``out`` and leaves h alone.
-    y [T, H] in the activations' type or float; None: only shift and norm."""
+    y [T, H] in the activations' type or float; None: only shift and norm.
+    ``conv`` = (w, state, slots, positions), as ``short_conv`` takes them, for a step in which every
+    row is a request of its own that brings one token: the normed rows then pass the short
+    convolution in the same kernel (``branch_join_takes_conv`` says for which sizes)."""
     _dev(h, y, branch_weight, shift, next_weight, out, rows)
     _f32(branch_weight, shift, next_weight)
+    cw = cstate = cslots = cpos = None
+    taps = 1
+    if conv is not None:
+        cw, cstate, cslots, cpos = conv
+        _dev(cw, cstate, cslots, cpos)
+        _f32(cw)
+        taps = cw.shape[1]
+        if not branch_join_takes_conv(h.shape[1]) or rows is not None or next_weight is None or \
+                tuple(cw.shape) != (h.shape[1], taps) or cslots.numel() != h.shape[0] or cpos.numel() != h.shape[0] or \
+                (taps > 1 and (cstate is None or cstate.dtype != out.dtype or tuple(cstate.shape[1:]) != (taps - 1, h.shape[1]))):
+            raise KernelError("branch_join: the convolution's operands do not fit the step")
     T, H = h.shape
     n = T if rows is None else rows.numel()
     if h.dtype != torch.float32 or (y is not None and (tuple(y.shape) != (T, H) or branch_weight is None or
@@ -870,8 +888,14 @@ def branch_join(h: torch.Tensor, y: torch.Tensor | None, branch_weight: torch.Te
     lib = core()
     _check(lib.lyp_branch_join(_p(h), _p(y), _code(y.dtype) if y is not None else 0, _p(branch_weight), float(mult),
                                _p(shift), _p(next_weight), _p(out), _code(out.dtype) if out is not None else 0,
-                               _p(rows), n, H, float(eps_branch), float(eps_next), _stream()), lib)
+                               _p(rows), n, H, float(eps_branch), float(eps_next), _p(cw), _p(cstate), _p(cslots),
+                               _p(cpos), taps, _stream()), lib)
     return out
+
+
+def branch_join_takes_conv(H: int) -> bool:
+    """Whether ``branch_join`` can carry the short convolution of a decode step's rows of H values."""
+    return H % 4 == 0 and H <= 16384
 
 
 def add_row(h: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
@@ -925,9 +949,13 @@ def activation(x: torch.Tensor, kind: str, params: torch.Tensor | None = None,
 
 
 def mingru_scan(pre: torch.Tensor, bz: torch.Tensor, bx: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor,
-                positions: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, B: int) -> torch.Tensor:
+                positions: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, B: int,
+                workspace: torch.Tensor | None = None) -> torch.Tensor:
     """The minGRU recurrence over the step's rows, request by request: pre float [T, 3 W] holds the
-    update-gate, candidate and output-gate projections side by side; state float [slots, W]."""
+    update-gate, candidate and output-gate projections side by side; state float [slots, W].
+    Without a workspace a thread walks all rows of its request and channel (steps of few rows per
+    request); with one (``mingru_scan_workspace`` floats) the rows go in chunks of 64 that run side by
+    side: a pass for every chunk's summary, a pass for the outputs (the recurrence is linear in the state)."""
     _dev(pre, bz, bx, state, q_start, positions, slots, out)
     _f32(pre, bz, bx, state)
     T, W = out.shape
@@ -935,9 +963,23 @@ def mingru_scan(pre: torch.Tensor, bz: torch.Tensor, bx: torch.Tensor, state: to
             q_start.numel() != B + 1 or slots.numel() != B or positions.numel() != T:
         raise KernelError(f"mingru_scan: pre {tuple(pre.shape)}, out {tuple(out.shape)}, state {tuple(state.shape)}")
     lib = core()
+    if workspace is not None:
+        _dev(workspace)
+        _f32(workspace)
+        if workspace.numel() < mingru_scan_workspace(T, B, W):
+            raise KernelError("mingru_scan: workspace too small")
+        _check(lib.lyp_mingru_scan_chunks(_p(pre), _p(bz), _p(bx), _p(state), _p(q_start), _p(positions), _p(slots),
+                                          _p(out), _code(out.dtype), T, B, W, _p(workspace), workspace.numel(),
+                                          _stream()), lib)
+        return out
     _check(lib.lyp_mingru_scan(_p(pre), _p(bz), _p(bx), _p(state), _p(q_start), _p(positions), _p(slots), _p(out),
                                _code(out.dtype), B, W, _stream()), lib)
     return out
+
+
+def mingru_scan_workspace(T: int, B: int, W: int) -> int:
+    """Floats of the workspace with which ``mingru_scan`` walks a step's rows in chunks of 64."""
+    return (2 * (-(-T // 64) + B) + B) * W
 
 
 def latent_prep(d: torch.Tensor, wq: torch.Tensor, wkv: torch.Tensor, positions: torch.Tensor,

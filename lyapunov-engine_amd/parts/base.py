@@ -351,6 +351,11 @@ class InputFilter(Part):
     def state_spec(self) -> Optional[StateSpec]:
         return None
 
+    def fused(self, ctx: StepContext, state: Optional[torch.Tensor], width: int):
+        """Operands with which the norm in front of the filter can run it in its own kernel, for a
+        step in which every request brings one token; None: the filter runs by itself."""
+        return None
+
     def forward(self, ctx: StepContext, x: torch.Tensor, state: Optional[torch.Tensor]) -> torch.Tensor:
         raise NotImplementedError
 

@@ -76,9 +76,17 @@ class SandwichBlock(Block):
         return {"filter": st} if st is not None else {}
 
     def forward(self, ctx: StepContext, h, delta, cache: LayerCache):
-        x = normed(self.norm1, None, ctx, h, delta)
-        if self.filter is not None:
-            x = self.filter.forward(ctx, x, cache.states.get("filter"))
+        conv = None
+        if self.filter is not None and ctx.T == ctx.B and (delta is None or isinstance(delta, ops.JoiningBranch)) \
+                and getattr(self.norm1, "joins_branches", False):
+            # every request brings one token: the filter rides in the norm's kernel
+            conv = self.filter.fused(ctx, cache.states.get("filter"), self.norm1.size)
+        if conv is not None:
+            x = self.norm1.forward(ctx, h, delta, conv=conv)
+        else:
+            x = normed(self.norm1, None, ctx, h, delta)
+            if self.filter is not None:
+                x = self.filter.forward(ctx, x, cache.states.get("filter"))
         branch = self.norm1_out.branch(self.mixer.forward(ctx, x, cache), self.mult)
         if self.ffn is None:
             return h, branch

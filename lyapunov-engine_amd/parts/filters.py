@@ -36,6 +36,13 @@ class CausalShortConv(InputFilter):
         # the inputs are activations; they are kept as they were read
         return StateSpec((self.taps - 1, self.channels), None) if self.taps > 1 else None
 
+    def fused(self, ctx: StepContext, state: Optional[torch.Tensor], width: int):
+        """What ``ops.branch_join`` needs to run this filter behind a norm in one kernel (a step
+        in which every request brings one token), or None where it cannot."""
+        if not self.residual or width != self.channels or not ops.branch_join_takes_conv(width):
+            return None
+        return (self.weight_f, state, ctx.state_slots, ctx.positions)
+
     def forward(self, ctx: StepContext, x: torch.Tensor, state: Optional[torch.Tensor]) -> torch.Tensor:
         out = torch.empty_like(x)
         return ops.short_conv(x, self.weight_f, state, ctx.q_start, ctx.positions, ctx.state_slots, out, ctx.B,

@@ -125,7 +125,8 @@ class LatentAttention(Mixer):
         ops.latent_query_rotate(q, ctx.positions, table, qa, num_heads=H, dim=self.dim, rot_dim=self.rot_dim,
                                 kv_rank=self.kv_rank)
         # a recorded step may hold rows that belong to no request: nothing writes them
-        mixed = (torch.zeros if ctx.fixed is not None else torch.empty)((T, H, self.kv_rank), dtype=ctx.dtype, device=dev)
+        padded_rows = ctx.fixed is not None and ctx.fixed.tokens > 0
+        mixed = (torch.zeros if padded_rows else torch.empty)((T, H, self.kv_rank), dtype=ctx.dtype, device=dev)
         if self.matrix_cores:
             launch = ops.latent_attn_launch(T, ctx.B, H, ctx.plans[ContextBound.key].meta["max_ctx"], ctx.dtype,
                                             self.kv_rank, self.rot_dim)

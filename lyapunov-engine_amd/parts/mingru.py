@@ -30,6 +30,8 @@ class MinGRU(Mixer):
         self.z_bias = self.x_bias = self.out_proj = None
         self.z_bias_f = self.x_bias_f = None
 
+    CHUNKED_FROM = 32   # mean rows per request from which the scan runs in chunks
+
     def weight_specs(self):
         n, shape = self.names, (self.width, self.hidden_size)
         return [
@@ -49,6 +51,9 @@ class MinGRU(Mixer):
     def forward(self, ctx: StepContext, x, cache: LayerCache):
         pre = ops.linear(x, self.in_proj, out_dtype=torch.float32)
         gated = torch.empty((ctx.T, self.width), dtype=ctx.dtype, device=pre.device)
+        # long runs of rows go in chunks side by side; a step of few rows per request walks them in order
+        ws = ctx.scratch("mingru_chunks", ops.mingru_scan_workspace(ctx.T, ctx.B, self.width)) \
+            if ctx.T > self.CHUNKED_FROM * ctx.B else None
         ops.mingru_scan(pre, self.z_bias_f, self.x_bias_f, cache.state, ctx.q_start, ctx.positions, ctx.state_slots,
-                        gated, ctx.B)
+                        gated, ctx.B, ws)
         return ops.linear(gated, self.out_proj, out_dtype=ctx.dtype)

@@ -53,12 +53,17 @@ class RMSNorm(Norm):
     # ops.PendingNorm for the consumer's kernel to norm on its way in.
     can_defer = True
 
-    def forward(self, ctx: StepContext, h, delta=None, rows=None, lazy=False):
-        if isinstance(delta, ops.JoiningBranch):
+    def forward(self, ctx: StepContext, h, delta=None, rows=None, lazy=False, conv=None):
+        """``conv``: see ``ops.branch_join``; the caller has checked that it applies (delta None or a
+        joining branch, every row a request of one token, sizes that ``ops.branch_join_takes_conv``)."""
+        if isinstance(delta, ops.JoiningBranch) or conv is not None:
             n = h.shape[0] if rows is None else rows.numel()
             out = torch.empty((n, self.size), dtype=ctx.dtype, device=h.device)
+            if delta is None:
+                return ops.branch_join(h, None, None, 1.0, 0.0, next_weight=self.weight_f, eps_next=self.eps, out=out,
+                                       rows=rows, conv=conv)
             return ops.branch_join(h, delta.y, delta.weight, delta.mult, delta.eps, shift=delta.shift,
-                                   next_weight=self.weight_f, eps_next=self.eps, out=out, rows=rows)
+                                   next_weight=self.weight_f, eps_next=self.eps, out=out, rows=rows, conv=conv)
         if lazy and rows is None:
             pending, delta = ops.rmsnorm_pending(h, self.weight, self.eps, ctx.dtype, delta)
             if pending is not None:

@@ -123,7 +123,42 @@ def test_activations(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_mingru_scan_in_portions(dtype):
+@pytest.mark.parametrize("taps", [1, 2, 4])
+def test_norm_and_filter_in_one_kernel_for_steps_of_single_tokens(dtype, taps):
+    """Three requests decode side by side for ten steps (one starts later, in a slot with stale
+    contents): join, norm and filter in one kernel against the plain functions on whole sequences."""
+    from lyapunov_engine_amd.kernels import ops
+
+    H, n = 136, 10
+    g = torch.Generator().manual_seed(taps)
+    w = torch.randn(H, taps, generator=g)
+    wn, wb = 1 + 0.2 * torch.randn(H, generator=g), 1 + 0.2 * torch.randn(H, generator=g)
+    hs = torch.randn(3, n, H, generator=g)
+    ys = torch.randn(3, n, H, generator=g).to(tdt(dtype))
+    state = torch.full((4, max(taps - 1, 1), H), 55.0, dtype=tdt(dtype), device=DEV)[:, :taps - 1].contiguous() if taps > 1 else None
+    want = []
+    for r in range(3):
+        joined = hs[r].double() + 0.5 * FP.rms_norm(ys[r].double(), wb.double(), 1e-5)
+        x = FP.rms_norm(joined, wn.double(), 1e-6)
+        if dtype == "bfloat16":
+            x = x.to(torch.bfloat16).double()          # the filter reads activations
+        want.append(x + FP.short_conv(x, w.double()))
+    for t in range(n):
+        live = [0, 1] if t < 3 else [0, 1, 2]            # request 2 starts at step 3, at its own position 0
+        pos = [t, t] if t < 3 else [t, t, t - 3]
+        h = torch.stack([hs[r, p] for r, p in zip(live, pos)]).to(DEV)
+        y = torch.stack([ys[r, p] for r, p in zip(live, pos)]).to(DEV)
+        to = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
+        out = torch.empty(len(live), H, dtype=tdt(dtype), device=DEV)
+        ops.branch_join(h, y, wb.to(DEV), 0.5, 1e-5, next_weight=wn.to(DEV), eps_next=1e-6, out=out,
+                        conv=(w.to(DEV), state, to([3, 0, 2][:len(live)]), to(pos)))
+        for i, (r, p) in enumerate(zip(live, pos)):
+            close(out[i], want[r][p], dtype, f"taps {taps} step {t} request {r}")
+
+
+@pytest.mark.parametrize("chunked", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_mingru_scan_in_portions(dtype, chunked):
     from lyapunov_engine_amd.kernels import ops
 
     W = 100
@@ -149,7 +184,8 @@ def test_mingru_scan_in_portions(dtype):
         x = torch.cat([pre[r][fed[r]:fed[r] + n] for r, n in step]).to(DEV)
         q_start, pos, slots = step_tables([n for _, n in step], [fed[r] for r, _ in step], [3 if r == "a" else 1 for r, _ in step])
         out = torch.empty(x.shape[0], W, dtype=tdt(dtype), device=DEV)
-        ops.mingru_scan(x, bz.to(DEV), bx.to(DEV), state, q_start, pos, slots, out, len(step))
+        ws = torch.full((ops.mingru_scan_workspace(x.shape[0], len(step), W),), float("nan"), device=DEV) if chunked else None
+        ops.mingru_scan(x, bz.to(DEV), bx.to(DEV), state, q_start, pos, slots, out, len(step), ws)
         at = 0
         for r, n in step:
             close(out[at:at + n], want[r][fed[r]:fed[r] + n], dtype, f"request {r} from {fed[r]}")
