@@ -12,7 +12,8 @@
 // Work: the (token, head) pairs of a request, flattened token by token, are cut
 // into groups of 64 rows; a workgroup of four waves takes one group (16 rows a
 // wave) and one partition of the keys.  All four waves load a tile of keys into
-// LDS together; each then computes, per 16 keys,
+// LDS together, row by row for the scores and transposed for the sums; each then
+// computes, per 32 keys in bfloat16 (16x16x32 instructions) and per 16 in float,
 //     S^T = K Q^T          (keys x rows; the accumulator leaves every lane with one
 //                           row's scores for four keys, which is the operand layout
 //                           of the next product, so the weights never leave registers)
@@ -39,13 +40,20 @@ constexpr int DK = KV + RD;
 static_assert(KV % 16 == 0 && RD % 16 == 0 && KV > 0, "latent sizes in multiples of 16");
 constexpr int kRowsPerGroup = 64;
 
+// LDS of a workgroup: a tile of keys row by row (Kr, for the scores) and the same tile's first KV
+// columns transposed (Vt[dimension][key], for the sums), so that both products read their operand
+// along the dimension they add over.  Vt's groups of four keys are stored at (group ^ dimension %
+// groups): the sums' reads (16 lanes, 16 neighbouring dimensions, one group) then fall on different
+// banks.
 template <typename T>
 struct Tile {
   static constexpr int kPad = 16 / sizeof(T);
-  static constexpr int kLd = DK + kPad;
-  // keys staged per round: as many as 48 KiB of LDS hold, 16 to 64
-  static constexpr int kKeys = (kLd * sizeof(T) * 64 <= 48 * 1024) ? 64 : ((kLd * sizeof(T) * 32 <= 48 * 1024) ? 32 : 16);
-  static constexpr size_t kBytes = static_cast<size_t>(kKeys) * kLd * sizeof(T);
+  static constexpr int kLdK = DK + kPad;
+  static constexpr size_t bytes(int keys) { return (static_cast<size_t>(keys) * kLdK + static_cast<size_t>(KV) * keys) * sizeof(T); }
+  // keys staged per round: as many as 80 KiB of LDS hold, 64 or 32
+  static constexpr int kKeys = bytes(64) <= 80 * 1024 ? 64 : 32;
+  static constexpr size_t kBytes = bytes(kKeys);
+  static_assert(kBytes <= 160 * 1024, "a tile of 32 keys must fit the LDS");
 };
 
 template <typename T>
@@ -54,17 +62,23 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
     int page_size, const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ ctx_len, int B, const float* __restrict__ sink, float scale, T* __restrict__ out,
     float* __restrict__ part_o, float* __restrict__ part_ml, int H, int n_parts, int part_keys) {
-  using M = Mma16<T>;
-  using Frag = typename M::Frag;
-  constexpr int LD = Tile<T>::kLd;
+  using MW = Mma16Wide<T>;                 // 16 x 16 tile over KCH values of the inner dimension
+  using WFrag = typename MW::Frag;
+  using M4 = Mma16<T>;                     // the same over 16 values (four a lane)
+  using Frag = typename M4::Frag;
+  constexpr int KE = MW::kElems;           // inner-dimension values a lane holds: 8 (bfloat16) or 4 (float)
+  constexpr int KCH = 4 * KE;              // inner-dimension values per instruction: 32 or 16
+  constexpr int NS = KE / 4;               // 16-key subtiles per step of the sums: 2 or 1
+  constexpr int LDK = Tile<T>::kLdK;
   constexpr int KT = Tile<T>::kKeys;
-  constexpr int NC = DK / 16;   // chunks of the key dimension
-  constexpr int NV = KV / 16;   // chunks of the value dimension
-  constexpr int VEC = 16 / sizeof(T);
-  constexpr int VPR = DK / VEC;  // 16-byte vectors per key row
-  typedef T VecT __attribute__((ext_vector_type(VEC)));
+  constexpr int NQ = KT / 4;               // groups of four keys in a tile
+  constexpr int NCW = DK / KCH;            // full chunks of the key dimension
+  constexpr bool TAIL = DK % KCH != 0;     // 16 more values (bfloat16 with DK = 32 n + 16)
+  constexpr int NV = KV / 16;              // chunks of the value dimension
+  constexpr int DQ = DK / 4;               // groups of four dimensions in a key row
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  T* Ks = reinterpret_cast<T*>(smem_raw);
+  T* Kr = reinterpret_cast<T*>(smem_raw);
+  T* Vt = Kr + KT * LDK;
 
   // which request and which group of its rows
   int rem = blockIdx.x, b = 0, rows_b = 0;
@@ -98,16 +112,21 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
   const int wave_last = min(row0 + wave * 16 + 16, rows_b) - 1;
   const int wave_end = (live && wave_last >= row0 + wave * 16) ? positions[q0 + wave_last / H] + 1 : 0;
 
-  Frag qf[NC];
+  WFrag qf[NCW > 0 ? NCW : 1];
+  Frag qtail;
   {
     const T* qrow = qa + grow * DK;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      if (valid) qf[c] = *reinterpret_cast<const Frag*>(qrow + c * 16 + 4 * grp);
+    for (int c = 0; c < NCW; ++c) {
+      if (valid) qf[c] = *reinterpret_cast<const WFrag*>(qrow + c * KCH + KE * grp);
       else
 #pragma unroll
-        for (int e = 0; e < 4; ++e) qf[c][e] = from_f32<T>(0.f);
+        for (int e = 0; e < KE; ++e) qf[c][e] = from_f32<T>(0.f);
     }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) qtail[e] = from_f32<T>(0.f);
+    if constexpr (TAIL)
+      if (valid) qtail = *reinterpret_cast<const Frag*>(qrow + NCW * KCH + 4 * grp);
   }
   f32x4 o[NV];
 #pragma unroll
@@ -117,66 +136,100 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
   const int32_t* table = block_tables + static_cast<size_t>(b) * table_width;
   for (int k0 = k_begin; k0 < k_end; k0 += KT) {
     __syncthreads();   // the tile before this one has been used by every wave
-    for (int idx = tid; idx < KT * VPR; idx += 256) {
-      const int j = idx / VPR, v = idx % VPR;
-      const int key = k0 + j;
-      VecT val;
+    // a thread a group of four keys x four dimensions: four loads, four row writes, four transposed writes
+    for (int idx = tid; idx < NQ * DQ; idx += 256) {
+      const int kq = idx / DQ, dq = idx % DQ;
+      Frag f[4];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) val[e] = from_f32<T>(0.f);
-      if (key < k_end) {
-        const int page = table[key / page_size];
-        if (page >= 0)
-          val = *reinterpret_cast<const VecT*>(pages + (static_cast<size_t>(page) * page_size + key % page_size) * DK +
-                                               v * VEC);
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[i][e] = from_f32<T>(0.f);
+        const int key = k0 + 4 * kq + i;
+        if (key < k_end) {
+          const int page = table[key / page_size];
+          if (page >= 0)
+            f[i] = *reinterpret_cast<const Frag*>(pages + (static_cast<size_t>(page) * page_size + key % page_size) * DK +
+                                                  4 * dq);
+        }
       }
-      *reinterpret_cast<VecT*>(Ks + j * LD + v * VEC) = val;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<Frag*>(Kr + (4 * kq + i) * LDK + 4 * dq) = f[i];
+      if (4 * dq < KV) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int d = 4 * dq + e;
+          Frag t;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) t[i] = f[i][e];
+          *reinterpret_cast<Frag*>(Vt + d * KT + 4 * (kq ^ (d % NQ))) = t;
+        }
+      }
     }
     __syncthreads();
     const int tile_end = min(KT, k_end - k0);
-    for (int kk = 0; kk < tile_end; kk += 16) {
+    for (int kk = 0; kk < tile_end; kk += 16 * NS) {
       if (k0 + kk >= wave_end) break;   // nothing further is seen by this wave's rows
-      f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
-      const T* krow = Ks + (kk + col) * LD + 4 * grp;
-#pragma unroll
-      for (int c = 0; c < NC; ++c) s = M::mma(*reinterpret_cast<const Frag*>(krow + c * 16), qf[c], s);
-      // s[e]: score of key k0 + kk + 4 grp + e for row `col`
+      f32x4 s[NS];
       float tmax = LYP_NEG_INF;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int key = k0 + kk + 4 * grp + e;
-        s[e] = key < limit ? s[e] * scale : LYP_NEG_INF;
-        tmax = fmaxf(tmax, s[e]);
+      for (int u = 0; u < NS; ++u) {
+        s[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const T* krow = Kr + (kk + 16 * u + col) * LDK;
+#pragma unroll
+        for (int c = 0; c < NCW; ++c)
+          s[u] = MW::mma(*reinterpret_cast<const WFrag*>(krow + c * KCH + KE * grp), qf[c], s[u]);
+        if constexpr (TAIL) {   // the last 16 values in a product of their own, added afterwards
+          const f32x4 t = M4::mma(*reinterpret_cast<const Frag*>(krow + NCW * KCH + 4 * grp), qtail,
+                                  f32x4{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[u][e] += t[e];
+        }
+        // s[u][e]: score of key k0 + kk + 16 u + 4 grp + e for row `col`
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = k0 + kk + 16 * u + 4 * grp + e;
+          s[u][e] = key < limit ? s[u][e] * scale : LYP_NEG_INF;
+          tmax = fmaxf(tmax, s[u][e]);
+        }
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
       const float m_new = fmaxf(m, tmax);
       float alpha = 1.f, psum = 0.f;
-      Frag pf;
+      WFrag pf;
       if (m_new > LYP_NEG_INF) {
         alpha = expf(m - m_new);   // m = -inf: 0
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float p = expf(s[e] - m_new);
-          psum += p;
-          pf[e] = from_f32<T>(p);
-        }
+        for (int u = 0; u < NS; ++u)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float p = expf(s[u][e] - m_new);
+            psum += p;
+            pf[4 * u + e] = from_f32<T>(p);
+          }
       } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) pf[e] = from_f32<T>(0.f);
+        for (int e = 0; e < KE; ++e) pf[e] = from_f32<T>(0.f);
       }
       psum += __shfl_xor(psum, 16, kWave);
       psum += __shfl_xor(psum, 32, kWave);
       l = l * alpha + psum;
       m = m_new;
-      const T* vbase = Ks + (kk + 4 * grp) * LD + col;
+      const int quad = kk / 4 + grp;
 #pragma unroll
       for (int v = 0; v < NV; ++v) {
-        Frag vf;
+        const int d = v * 16 + col;
+        const T* vrow = Vt + d * KT;
+        WFrag vf;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) vf[e] = vbase[e * LD + v * 16];
+        for (int u = 0; u < NS; ++u) {
+          const Frag piece = *reinterpret_cast<const Frag*>(vrow + 4 * ((quad + 4 * u) ^ (d % NQ)));
+#pragma unroll
+          for (int e = 0; e < 4; ++e) vf[4 * u + e] = piece[e];
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[v][e] *= alpha;
-        o[v] = M::mma(vf, pf, o[v]);
+        o[v] = MW::mma(vf, pf, o[v]);
       }
     }
   }
@@ -192,15 +245,16 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
       inv = 1.0f / (l * w + expf(sk - mx));
     }
 #pragma unroll
-    for (int v = 0; v < NV; ++v)
+    for (int v = 0; v < NV; ++v) {
+      Frag res;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) orow[v * 16 + 4 * grp + e] = from_f32<T>(valid ? o[v][e] * w * inv : 0.f);
+      for (int e = 0; e < 4; ++e) res[e] = from_f32<T>(valid ? o[v][e] * w * inv : 0.f);
+      *reinterpret_cast<Frag*>(orow + v * 16 + 4 * grp) = res;
+    }
   } else {
     float* prow = part_o + (grow * n_parts + part) * KV;
 #pragma unroll
-    for (int v = 0; v < NV; ++v)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) prow[v * 16 + 4 * grp + e] = o[v][e];
+    for (int v = 0; v < NV; ++v) *reinterpret_cast<f32x4*>(prow + v * 16 + 4 * grp) = o[v];
     if (grp == 0) {
       part_ml[(grow * n_parts + part) * 2] = valid ? m : LYP_NEG_INF;
       part_ml[(grow * n_parts + part) * 2 + 1] = valid ? l : 0.f;

@@ -27,10 +27,11 @@ def tdt(dtype):
     return torch.float32 if dtype == "float32" else torch.bfloat16
 
 
-def close(got, want, dtype, what=""):
+def close(got, want, dtype, what="", floor=1.0):
+    """Largest difference against ``tol`` times the largest wanted value (at least ``floor``)."""
     got, want = got.double().cpu(), want.double().cpu()
     tol = 2e-5 if dtype == "float32" else 2e-2
-    scale = max(1.0, float(want.abs().max()))
+    scale = max(floor, float(want.abs().max()))
     err = float((got - want).abs().max())
     assert err <= tol * scale, f"{what}: max error {err:.3e} at scale {scale:.3f}"
 
@@ -265,7 +266,8 @@ def test_latent_attention_over_pages(dtype, shape, kernel):
     keys, qa, sink = latent_case(dtype, T_ctx, H, kv_rank, rot_dim, page_size, seed=T_ctx, n_new=n_new)
     scale = (kv_rank + rot_dim) ** -0.5
     got = run_latent_attention(dtype, keys, qa, sink, scale, kv_rank, rot_dim, page_size, kernel=kernel)
-    close(got, plain_latent_attention(keys, qa, sink, scale, kv_rank), dtype, f"latent attention {shape}")
+    # sums over hundreds of keys are small: held to their own size, not to 1
+    close(got, plain_latent_attention(keys, qa, sink, scale, kv_rank), dtype, f"latent attention {shape}", floor=1e-3)
 
 
 @pytest.mark.parametrize("kernel", KERNELS)
@@ -283,6 +285,26 @@ def test_latent_attention_finds_one_planted_key(dtype, where, kernel):
     want = plain_latent_attention(keys, qa, sink, 1.0, kv_rank)
     close(got, want, dtype, f"planted key at {where}")
     assert torch.allclose(want[0, 0], keys[where, :kv_rank].double(), atol=0.05), "the planted key must carry the result"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("sizes", [(16, 0), (16, 16), (32, 16), (48, 0), (16, 32), (64, 16), (32, 48), (96, 16), (64, 64),
+                                   (128, 16), (128, 32)])
+def test_matrix_core_kernel_finds_planted_keys_at_every_size(dtype, sizes):
+    """The matrix-core kernel walks the key dimension in instructions of 32 and of 16 values, by
+    sizes: every combination has to find a planted key at every place of a tile (with eight
+    dimensions of a score missing, a planted key would still win most of the time, so all places of
+    two tiles are tried)."""
+    kv_rank, rot_dim = sizes
+    T_ctx, H, page_size = 130, 3, 16
+    keys, _, _ = latent_case(dtype, T_ctx, H, kv_rank, rot_dim, page_size, seed=kv_rank + rot_dim, n_new=1)
+    keys = (keys.float() * 0.1).to(tdt(dtype))
+    sink = torch.full((H,), -50.0)
+    for where in range(0, T_ctx, 3):
+        qa = (keys[where].float() * (19200.0 / (kv_rank + rot_dim)))[None, None, :].repeat(1, H, 1).to(tdt(dtype))
+        got = run_latent_attention(dtype, keys, qa, sink, 1.0, kv_rank, rot_dim, page_size, kernel="cores")
+        want = plain_latent_attention(keys, qa, sink, 1.0, kv_rank)
+        close(got, want, dtype, f"sizes {sizes}, planted key at {where}", floor=1e-3)
 
 
 @pytest.mark.parametrize("kernel", KERNELS)
