@@ -42,9 +42,8 @@ constexpr int kRowsPerGroup = 64;
 
 // LDS of a workgroup: a tile of keys row by row (Kr, for the scores) and the same tile's first KV
 // columns transposed (Vt[dimension][key], for the sums), so that both products read their operand
-// along the dimension they add over.  Vt's groups of four keys are stored at (group ^ dimension %
-// groups): the sums' reads (16 lanes, 16 neighbouring dimensions, one group) then fall on different
-// banks.
+// along the dimension they add over.  Vt's groups of four keys are stored at swizzled places
+// (swizzle below), which keeps reads and staging writes off each other's banks.
 template <typename T>
 struct Tile {
   static constexpr int kPad = 16 / sizeof(T);
@@ -56,12 +55,20 @@ struct Tile {
   static_assert(kBytes <= 160 * 1024, "a tile of 32 keys must fit the LDS");
 };
 
+// Where row d of Vt keeps its groups of four keys: group g stands at g ^ swizzle(d).  Both the
+// sums' reads (16 neighbouring rows, one group) and the staging writes (rows 4 i + e of 16
+// neighbouring i, one group) then fall on 16 different places.
+template <int NQ>
+__device__ __forceinline__ int swizzle(int d) {
+  return (d % NQ) ^ ((d / NQ) & 3);
+}
+
 template <typename T>
-__global__ __launch_bounds__(256) void latent_attn_kernel(
+__global__ __launch_bounds__(256, KV <= 256 ? 2 : 1) void latent_attn_kernel(
     const T* __restrict__ qa, const T* __restrict__ pages, const int32_t* __restrict__ block_tables, int table_width,
     int page_size, const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ ctx_len, int B, const float* __restrict__ sink, float scale, T* __restrict__ out,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int H, int n_parts, int part_keys) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, int H, int n_parts, int part_keys, int page_shift) {
   using MW = Mma16Wide<T>;                 // 16 x 16 tile over KCH values of the inner dimension
   using WFrag = typename MW::Frag;
   using M4 = Mma16<T>;                     // the same over 16 values (four a lane)
@@ -134,34 +141,67 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
   float m = LYP_NEG_INF, l = 0.f;
 
   const int32_t* table = block_tables + static_cast<size_t>(b) * table_width;
-  for (int k0 = k_begin; k0 < k_end; k0 += KT) {
-    __syncthreads();   // the tile before this one has been used by every wave
-    // a thread a group of four keys x four dimensions: four loads, four row writes, four transposed writes
-    for (int idx = tid; idx < NQ * DQ; idx += 256) {
-      const int kq = idx / DQ, dq = idx % DQ;
-      Frag f[4];
+  // Where a tile's keys lie in the pages (row numbers, -1 for none) is worked out a tile ahead by
+  // the first KT threads and kept in LDS, so that the loads of the keys themselves depend on no
+  // other load; a thread asks for all of its share of a tile at once (groups of four keys x four
+  // dimensions: four loads, four row writes, four transposed writes each).
+  __shared__ int rowidx[2][KT];
+  auto locate = [&](int k0, int buf) {
+    if (tid < KT) {
+      const int key = k0 + tid;
+      int row = -1;
+      if (key < k_end) {
+        const int page = page_shift >= 0 ? table[key >> page_shift] : table[key / page_size];
+        const int slot = page_shift >= 0 ? key & (page_size - 1) : key % page_size;
+        if (page >= 0) row = page * page_size + slot;
+      }
+      rowidx[buf][tid] = row;
+    }
+  };
+  constexpr int UNITS = NQ * DQ;
+  constexpr int TURNS = (UNITS + 255) / 256;
+  locate(k_begin, 0);
+  int buf = 0;
+  for (int k0 = k_begin; k0 < k_end; k0 += KT, buf ^= 1) {
+    __syncthreads();   // the tile before this one has been used by every wave; rowidx[buf] is written
+    // in rounds of up to three turns: the loads of a round are all asked for before the first is used
+    constexpr int ROUND = 3;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+    for (int t0 = 0; t0 < TURNS; t0 += ROUND) {
+      Frag stage[ROUND][4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) f[i][e] = from_f32<T>(0.f);
-        const int key = k0 + 4 * kq + i;
-        if (key < k_end) {
-          const int page = table[key / page_size];
-          if (page >= 0)
-            f[i] = *reinterpret_cast<const Frag*>(pages + (static_cast<size_t>(page) * page_size + key % page_size) * DK +
-                                                  4 * dq);
+      for (int t = 0; t < ROUND; ++t) {
+        const int idx = tid + (t0 + t) * 256;
+        const int kq = idx / DQ, dq = idx % DQ;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) stage[t][i][e] = from_f32<T>(0.f);
+          if (t0 + t < TURNS && idx < UNITS) {
+            const int row = rowidx[buf][4 * kq + i];
+            if (row >= 0)
+              stage[t][i] = *reinterpret_cast<const Frag*>(pages + static_cast<size_t>(row) * DK + 4 * dq);
+          }
         }
       }
+      if (t0 == 0 && k0 + KT < k_end) locate(k0 + KT, buf ^ 1);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<Frag*>(Kr + (4 * kq + i) * LDK + 4 * dq) = f[i];
-      if (4 * dq < KV) {
+      for (int t = 0; t < ROUND; ++t) {
+        const int idx = tid + (t0 + t) * 256;
+        if (t0 + t < TURNS && idx < UNITS) {
+          const int kq = idx / DQ, dq = idx % DQ;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int d = 4 * dq + e;
-          Frag t;
+          for (int i = 0; i < 4; ++i) *reinterpret_cast<Frag*>(Kr + (4 * kq + i) * LDK + 4 * dq) = stage[t][i];
+          if (4 * dq < KV) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) t[i] = f[i][e];
-          *reinterpret_cast<Frag*>(Vt + d * KT + 4 * (kq ^ (d % NQ))) = t;
+            for (int e = 0; e < 4; ++e) {
+              const int d = 4 * dq + e;
+              Frag tr;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) tr[i] = stage[t][i][e];
+              *reinterpret_cast<Frag*>(Vt + d * KT + 4 * (kq ^ swizzle<NQ>(d))) = tr;
+            }
+          }
         }
       }
     }
@@ -174,10 +214,16 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
 #pragma unroll
       for (int u = 0; u < NS; ++u) {
         s[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 s2 = f32x4{0.f, 0.f, 0.f, 0.f};   // odd chunks: two chains of dependent products instead of one
         const T* krow = Kr + (kk + 16 * u + col) * LDK;
 #pragma unroll
-        for (int c = 0; c < NCW; ++c)
-          s[u] = MW::mma(*reinterpret_cast<const WFrag*>(krow + c * KCH + KE * grp), qf[c], s[u]);
+        for (int c = 0; c < NCW; ++c) {
+          const WFrag kf = *reinterpret_cast<const WFrag*>(krow + c * KCH + KE * grp);
+          if (c % 2 == 0) s[u] = MW::mma(kf, qf[c], s[u]);
+          else s2 = MW::mma(kf, qf[c], s2);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[u][e] += s2[e];
         if constexpr (TAIL) {   // the last 16 values in a product of their own, added afterwards
           const f32x4 t = M4::mma(*reinterpret_cast<const Frag*>(krow + NCW * KCH + 4 * grp), qtail,
                                   f32x4{0.f, 0.f, 0.f, 0.f});
@@ -216,6 +262,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
       l = l * alpha + psum;
       m = m_new;
       const int quad = kk / 4 + grp;
+      const bool rescale = __any(alpha != 1.f);   // the sums are rescaled only when some row's maximum grew
 #pragma unroll
       for (int v = 0; v < NV; ++v) {
         const int d = v * 16 + col;
@@ -223,12 +270,13 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
         WFrag vf;
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
-          const Frag piece = *reinterpret_cast<const Frag*>(vrow + 4 * ((quad + 4 * u) ^ (d % NQ)));
+          const Frag piece = *reinterpret_cast<const Frag*>(vrow + 4 * ((quad + 4 * u) ^ swizzle<NQ>(d)));
 #pragma unroll
           for (int e = 0; e < 4; ++e) vf[4 * u + e] = piece[e];
         }
+        if (rescale)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[v][e] *= alpha;
+          for (int e = 0; e < 4; ++e) o[v][e] *= alpha;
         o[v] = MW::mma(vf, pf, o[v]);
       }
     }
@@ -264,7 +312,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
 
 // One wave per (token, head) row: merges the partitions' results and the sink.
 template <typename T>
-__global__ __launch_bounds__(64) void latent_combine_kernel(const float* __restrict__ part_o,
+__global__ __launch_bounds__(256) void latent_combine_kernel(const float* __restrict__ part_o,
                                                             const float* __restrict__ part_ml,
                                                             const float* __restrict__ sink, T* __restrict__ out,
                                                             int H, int n_parts) {
@@ -272,22 +320,28 @@ __global__ __launch_bounds__(64) void latent_combine_kernel(const float* __restr
   const size_t row = blockIdx.x;
   const int head = static_cast<int>(row % H);
   const float sk = sink[head];
-  // a lane a partition: maxima, weights and the denominator (partitions added in lane order)
-  float mx = sk;
-  for (int p = threadIdx.x; p < n_parts; p += kWave) mx = fmaxf(mx, part_ml[(row * n_parts + p) * 2]);
-  mx = wave_max(mx);
-  float part = 0.f;
-  for (int p = threadIdx.x; p < n_parts; p += kWave) {
-    const float mp = part_ml[(row * n_parts + p) * 2];
-    const float w = mp > LYP_NEG_INF ? expf(mp - mx) : 0.f;
-    weight[p] = w;
-    part += part_ml[(row * n_parts + p) * 2 + 1] * w;
+  __shared__ float denom_s;
+  // the first wave, a lane a partition: maxima, weights and the denominator (partitions added in
+  // lane order); then a thread a dimension
+  if (threadIdx.x < kWave) {
+    float mx = sk;
+    for (int p = threadIdx.x; p < n_parts; p += kWave) mx = fmaxf(mx, part_ml[(row * n_parts + p) * 2]);
+    mx = wave_max(mx);
+    float part = 0.f;
+    for (int p = threadIdx.x; p < n_parts; p += kWave) {
+      const float mp = part_ml[(row * n_parts + p) * 2];
+      const float w = mp > LYP_NEG_INF ? expf(mp - mx) : 0.f;
+      weight[p] = w;
+      part += part_ml[(row * n_parts + p) * 2 + 1] * w;
+    }
+    part = wave_sum(part);
+    if (threadIdx.x == 0) denom_s = part + expf(sk - mx);
   }
-  const float denom = wave_sum(part) + expf(sk - mx);
   __syncthreads();
-  const float inv = 1.0f / denom;
-  for (int d = threadIdx.x; d < KV; d += kWave) {
+  const float inv = 1.0f / denom_s;
+  for (int d = threadIdx.x; d < KV; d += blockDim.x) {
     float acc = 0.f;
+#pragma unroll 4
     for (int p = 0; p < n_parts; ++p) acc += part_o[(row * n_parts + p) * KV + d] * weight[p];
     out[row * KV + d] = from_f32<T>(acc * inv);
   }
@@ -334,6 +388,9 @@ int lyp_latent_attn(const void* qa, const void* pages, const int32_t* block_tabl
   LYP_REQUIRE(reinterpret_cast<uintptr_t>(qa) % 16 == 0 && reinterpret_cast<uintptr_t>(pages) % 16 == 0,
               "latent_attn: operands must be 16-byte aligned");
   if (n_rows == 0) return 0;
+  int page_shift = -1;
+  if ((page_size & (page_size - 1)) == 0)
+    for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
   dim3 grid(row_groups, n_parts);
 #define LYP_LATENT(T)                                                                                               \
   do {                                                                                                              \
@@ -345,10 +402,11 @@ int lyp_latent_attn(const void* qa, const void* pages, const int32_t* block_tabl
     }                                                                                                               \
     latent_attn_kernel<T><<<grid, 256, Tile<T>::kBytes, stream>>>(                                                  \
         static_cast<const T*>(qa), static_cast<const T*>(pages), block_tables, table_width, page_size, q_start,     \
-        positions, ctx_len, B, sink, scale, static_cast<T*>(out), part_o, part_ml, H, n_parts, part_keys);          \
+        positions, ctx_len, B, sink, scale, static_cast<T*>(out), part_o, part_ml, H, n_parts, part_keys,           \
+        page_shift);                                                                                                \
     if (n_parts > 1)                                                                                                \
-      latent_combine_kernel<T><<<n_rows * H, 64, 0, stream>>>(part_o, part_ml, sink, static_cast<T*>(out), H,       \
-                                                              n_parts);                                             \
+      latent_combine_kernel<T><<<n_rows * H, KV >= 256 ? 256 : (KV >= 128 ? 128 : 64), 0, stream>>>(                \
+          part_o, part_ml, sink, static_cast<T*>(out), H, n_parts);                                                 \
   } while (0)
   if (dtype == kF32) LYP_LATENT(float);
   else if (dtype == kBF16) LYP_LATENT(bf16_t);

@@ -96,13 +96,17 @@ __global__ void branch_join_vec_kernel(float* __restrict__ h, const TY* __restri
   f32x4* hrow = reinterpret_cast<f32x4*>(h + src * H);
   const Vec4Y* yrow = y ? reinterpret_cast<const Vec4Y*>(y + src * H) : nullptr;
   const int nvec = H / 4;
-  f32x4 hv[MAXV], yv[MAXV];
+  // every operand is asked for at the start: a step of few rows is as long as its chain of loads
+  f32x4 hv[MAXV], yv[MAXV], wbv[MAXV], shv[MAXV], wnv[MAXV];
   float ssy = 0.f;
 #pragma unroll
   for (int v = 0; v < MAXV; ++v) {
     const int idx = threadIdx.x + v * blockDim.x;
     if (idx < nvec) {
       hv[v] = hrow[idx];
+      if (yrow) wbv[v] = reinterpret_cast<const f32x4*>(wb)[idx];
+      if (shift) shv[v] = reinterpret_cast<const f32x4*>(shift)[idx];
+      if (w_next) wnv[v] = reinterpret_cast<const f32x4*>(w_next)[idx];
       if (yrow) {
         const Vec4Y t = yrow[idx];
 #pragma unroll
@@ -124,14 +128,12 @@ __global__ void branch_join_vec_kernel(float* __restrict__ h, const TY* __restri
     const int idx = threadIdx.x + v * blockDim.x;
     if (idx < nvec) {
       if (yrow) {
-        const f32x4 w = reinterpret_cast<const f32x4*>(wb)[idx];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) hv[v][i] += mult * ((yv[v][i] * inv_y) * w[i]);
+        for (int i = 0; i < 4; ++i) hv[v][i] += mult * ((yv[v][i] * inv_y) * wbv[v][i]);
       }
       if (shift) {
-        const f32x4 s = reinterpret_cast<const f32x4*>(shift)[idx];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) hv[v][i] += s[i];
+        for (int i = 0; i < 4; ++i) hv[v][i] += shv[v][i];
       }
       if (!rows && (yrow || shift)) hrow[idx] = hv[v];
 #pragma unroll
@@ -153,10 +155,9 @@ __global__ void branch_join_vec_kernel(float* __restrict__ h, const TY* __restri
   for (int v = 0; v < MAXV; ++v) {
     const int idx = threadIdx.x + v * blockDim.x;
     if (idx < nvec) {
-      const f32x4 w = reinterpret_cast<const f32x4*>(w_next)[idx];
       Vec4T o;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = from_f32<T>((hv[v][i] * inv) * w[i]);
+      for (int i = 0; i < 4; ++i) o[i] = from_f32<T>((hv[v][i] * inv) * wnv[v][i]);
       if constexpr (CONV) {
         float acc[4];
 #pragma unroll
