@@ -347,6 +347,61 @@ __global__ __launch_bounds__(256) void latent_combine_kernel(const float* __rest
   }
 }
 
+// For steps of few rows: the merge pass and the per-head value projection in one kernel.  One
+// workgroup per (token, head) row: the row of KV latent sums (merged from the partitions as
+// latent_combine_kernel does, or read from `mixed` when the keys were in one partition; rounded to
+// the activations' type either way, as the two-kernel path leaves it), then out[row, v] =
+// sum_r row[r] * w[head, v, r], a wave an output at a time, lanes over r.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_heads_out_kernel(const float* __restrict__ part_o,
+                                                               const float* __restrict__ part_ml,
+                                                               const float* __restrict__ sink,
+                                                               const T* __restrict__ mixed, const T* __restrict__ w,
+                                                               T* __restrict__ out, int H, int n_parts, int vdim) {
+  __shared__ float weight[256];
+  __shared__ float denom_s;
+  __shared__ float rowv[KV];
+  const size_t row = blockIdx.x;
+  const int head = static_cast<int>(row % H);
+  if (mixed) {
+    for (int d = threadIdx.x; d < KV; d += blockDim.x) rowv[d] = to_f32(mixed[row * KV + d]);
+  } else {
+    const float sk = sink[head];
+    if (threadIdx.x < kWave) {
+      float mx = sk;
+      for (int p = threadIdx.x; p < n_parts; p += kWave) mx = fmaxf(mx, part_ml[(row * n_parts + p) * 2]);
+      mx = wave_max(mx);
+      float part = 0.f;
+      for (int p = threadIdx.x; p < n_parts; p += kWave) {
+        const float mp = part_ml[(row * n_parts + p) * 2];
+        const float wgt = mp > LYP_NEG_INF ? expf(mp - mx) : 0.f;
+        weight[p] = wgt;
+        part += part_ml[(row * n_parts + p) * 2 + 1] * wgt;
+      }
+      part = wave_sum(part);
+      if (threadIdx.x == 0) denom_s = part + expf(sk - mx);
+    }
+    __syncthreads();
+    const float inv = 1.0f / denom_s;
+    for (int d = threadIdx.x; d < KV; d += blockDim.x) {
+      float acc = 0.f;
+#pragma unroll 4
+      for (int p = 0; p < n_parts; ++p) acc += part_o[(row * n_parts + p) * KV + d] * weight[p];
+      rowv[d] = to_f32(from_f32<T>(acc * inv));
+    }
+  }
+  __syncthreads();
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, waves = blockDim.x / kWave;
+  const T* wh = w + static_cast<size_t>(head) * vdim * KV;
+  for (int v = wave; v < vdim; v += waves) {
+    const T* wr = wh + static_cast<size_t>(v) * KV;
+    float acc = 0.f;
+    for (int r = lane; r < KV; r += kWave) acc += rowv[r] * to_f32(wr[r]);
+    acc = wave_sum(acc);
+    if (lane == 0) out[row * vdim + v] = from_f32<T>(acc);
+  }
+}
+
 }  // namespace lyp
 
 using namespace lyp;
@@ -371,13 +426,37 @@ int lyp_latent_plan(int row_groups, int max_ctx, int dtype) {
   return std::max(1, std::min(parts, 256));
 }
 
+// The merge of the partitions (or, with part_o == nullptr, the rows of `mixed` [rows, KV]) and the
+// per-head projection w [H, vdim, KV] -> out [rows, vdim]; rows = tokens * H.  For steps of few rows.
+int lyp_latent_heads_out(const float* part_o, const float* part_ml, const float* sink, const void* mixed,
+                         const void* w, void* out, int dtype, int rows, int H, int n_parts, int vdim,
+                         hipStream_t stream) {
+  LYP_REQUIRE(rows >= 0 && H > 0 && vdim > 0 && n_parts >= 1 && n_parts <= 256, "latent_heads_out: bad sizes");
+  LYP_REQUIRE((part_o != nullptr && part_ml != nullptr && sink != nullptr) != (mixed != nullptr),
+              "latent_heads_out: either the partitions or the merged rows");
+  if (rows == 0) return 0;
+  if (dtype == kF32)
+    latent_heads_out_kernel<float><<<rows, 256, 0, stream>>>(part_o, part_ml, sink, static_cast<const float*>(mixed),
+                                                             static_cast<const float*>(w), static_cast<float*>(out), H,
+                                                             n_parts, vdim);
+  else if (dtype == kBF16)
+    latent_heads_out_kernel<bf16_t><<<rows, 256, 0, stream>>>(part_o, part_ml, sink, static_cast<const bf16_t*>(mixed),
+                                                              static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out),
+                                                              H, n_parts, vdim);
+  else
+    LYP_REQUIRE(false, "latent_heads_out: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("latent_heads_out");
+  return 0;
+}
+
 // qa [rows, H, DK], pages [pages, page_size, DK], out [rows, H, KV] of dtype; tables as in a step.
+// merge == 0: with several partitions the merge pass is left to the caller (lyp_latent_heads_out).
 // row_groups: an upper bound on the 64-row groups of all requests (rows * H / 64 rounded up, plus one
 // per request).  n_parts > 1 needs part_o [rows * H * n_parts * KV] and part_ml [rows * H * n_parts * 2].
 int lyp_latent_attn(const void* qa, const void* pages, const int32_t* block_tables, int table_width, int page_size,
                     const int32_t* q_start, const int32_t* positions, const int32_t* ctx_len, int B,
                     const float* sink, float scale, void* out, int dtype, int n_rows, int H, int row_groups,
-                    int n_parts, int part_keys, float* part_o, float* part_ml, hipStream_t stream) {
+                    int n_parts, int part_keys, float* part_o, float* part_ml, int merge, hipStream_t stream) {
   LYP_REQUIRE(n_rows >= 0 && B > 0 && H > 0 && page_size > 0 && table_width > 0 && row_groups > 0,
               "latent_attn: bad sizes rows=%d B=%d H=%d page=%d", n_rows, B, H, page_size);
   LYP_REQUIRE(n_parts >= 1 && n_parts <= 256 && part_keys > 0, "latent_attn: %d partitions of %d keys", n_parts,
@@ -404,7 +483,7 @@ int lyp_latent_attn(const void* qa, const void* pages, const int32_t* block_tabl
         static_cast<const T*>(qa), static_cast<const T*>(pages), block_tables, table_width, page_size, q_start,     \
         positions, ctx_len, B, sink, scale, static_cast<T*>(out), part_o, part_ml, H, n_parts, part_keys,           \
         page_shift);                                                                                                \
-    if (n_parts > 1)                                                                                                \
+    if (n_parts > 1 && merge)                                                                                       \
       latent_combine_kernel<T><<<n_rows * H, KV >= 256 ? 256 : (KV >= 128 ? 128 : 64), 0, stream>>>(                \
           part_o, part_ml, sink, static_cast<T*>(out), H, n_parts);                                                 \
   } while (0)

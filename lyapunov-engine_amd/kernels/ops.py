@@ -1054,7 +1054,9 @@ def latent_lib(kv_rank: int, rot_dim: int) -> ctypes.CDLL:
         lib.lyp_latent_tile_keys.argtypes = [c_int]
         lib.lyp_latent_attn.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                         c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                        c_void_p, c_void_p, c_void_p]
+                                        c_void_p, c_void_p, c_int, c_void_p]
+        lib.lyp_latent_heads_out.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                             c_int, c_int, c_int, c_void_p]
         _latent[(kv_rank, rot_dim)] = lib
     return lib
 
@@ -1083,10 +1085,12 @@ def latent_attn_launch(T: int, B: int, H: int, max_ctx: int, dtype: torch.dtype,
 def latent_attn(qa: torch.Tensor, pages: torch.Tensor, block_tables: torch.Tensor, q_start: torch.Tensor,
                 positions: torch.Tensor, ctx_len: torch.Tensor, sink: torch.Tensor, scale: float, out: torch.Tensor,
                 launch: dict, part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None, *,
-                kv_rank: int, rot_dim: int) -> torch.Tensor:
+                kv_rank: int, rot_dim: int, merge: bool = True) -> torch.Tensor:
     """``latent_attn_rows`` on the matrix cores (sizes in multiples of 16), a prompt's rows and
     single tokens alike; ``launch`` comes from ``latent_attn_launch`` for a bound on the step's
-    contexts that the caller guarantees (keys beyond n_parts * part_keys would be left out)."""
+    contexts that the caller guarantees (keys beyond n_parts * part_keys would be left out).
+    ``merge=False``: with several partitions ``out`` is left unwritten and the partitions' results
+    stay in ``part_o`` / ``part_ml`` for ``latent_heads_out`` to merge."""
     _dev(qa, pages, block_tables, q_start, positions, ctx_len, sink, out, part_o, part_ml)
     _f32(sink, part_o, part_ml)
     T, H, Dk = qa.shape
@@ -1103,7 +1107,30 @@ def latent_attn(qa: torch.Tensor, pages: torch.Tensor, block_tables: torch.Tenso
     _check(lib.lyp_latent_attn(_p(qa), _p(pages), _p(block_tables), block_tables.shape[1], pages.shape[1], _p(q_start),
                                _p(positions), _p(ctx_len), B, _p(sink), float(scale), _p(out), _code(qa.dtype), T, H,
                                launch["row_groups"], launch["n_parts"], launch["part_keys"], _p(part_o), _p(part_ml),
-                               _stream()), lib)
+                               int(merge), _stream()), lib)
+    return out
+
+
+HEADS_OUT_MAX_ROWS = 512    # (token, head) rows up to which the merge and the value projection are one kernel
+
+
+def latent_heads_out(w: torch.Tensor, out: torch.Tensor, *, kv_rank: int, rot_dim: int, mixed: torch.Tensor | None = None,
+                     part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None,
+                     sink: torch.Tensor | None = None, n_parts: int = 1) -> torch.Tensor:
+    """For a step of few rows: out[t, h, :] = w[h] @ (the latent sums of row (t, h)), w [H, vdim,
+    kv_rank], the sums either merged here from the partitions ``latent_attn(..., merge=False)``
+    left (with the sink), or read from ``mixed`` [T, H, kv_rank]."""
+    _dev(w, out, mixed, part_o, part_ml, sink)
+    _f32(part_o, part_ml, sink)
+    T, H, vdim = out.shape
+    if tuple(w.shape) != (H, vdim, kv_rank) or w.dtype != out.dtype or (mixed is None) == (part_o is None) or \
+            (mixed is not None and (tuple(mixed.shape) != (T, H, kv_rank) or mixed.dtype != out.dtype)) or \
+            (part_o is not None and (part_ml is None or sink is None or part_o.numel() < T * H * n_parts * kv_rank
+                                     or part_ml.numel() < T * H * n_parts * 2 or sink.numel() != H)):
+        raise KernelError(f"latent_heads_out: w {tuple(w.shape)}, out {tuple(out.shape)}")
+    lib = latent_lib(kv_rank, rot_dim)
+    _check(lib.lyp_latent_heads_out(_p(part_o), _p(part_ml), _p(sink), _p(mixed), _p(w), _p(out), _code(out.dtype),
+                                    T * H, H, n_parts, vdim, _stream()), lib)
     return out
 
 

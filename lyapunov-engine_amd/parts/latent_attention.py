@@ -127,6 +127,7 @@ class LatentAttention(Mixer):
         # a recorded step may hold rows that belong to no request: nothing writes them
         padded_rows = ctx.fixed is not None and ctx.fixed.tokens > 0
         mixed = (torch.zeros if padded_rows else torch.empty)((T, H, self.kv_rank), dtype=ctx.dtype, device=dev)
+        heads = torch.empty((T, H, self.vdim), dtype=ctx.dtype, device=dev)
         if self.matrix_cores:
             launch = ops.latent_attn_launch(T, ctx.B, H, ctx.plans[ContextBound.key].meta["max_ctx"], ctx.dtype,
                                             self.kv_rank, self.rot_dim)
@@ -134,11 +135,19 @@ class LatentAttention(Mixer):
             if launch["n_parts"] > 1:
                 part_o = ctx.scratch("latent_part_o", launch["part_o"])
                 part_ml = ctx.scratch("latent_part_ml", launch["part_ml"])
+            few = T * H <= ops.HEADS_OUT_MAX_ROWS and not padded_rows
             ops.latent_attn(qa, pages, g.block_tables, ctx.q_start, ctx.positions, ctx.ctx_len, self.sink_f,
-                            self.scale, mixed, launch, part_o, part_ml, kv_rank=self.kv_rank, rot_dim=self.rot_dim)
+                            self.scale, mixed, launch, part_o, part_ml, kv_rank=self.kv_rank, rot_dim=self.rot_dim,
+                            merge=not few)
+            if few:   # few rows: the partitions' merge and the heads' value projection in one kernel
+                if launch["n_parts"] > 1:
+                    ops.latent_heads_out(self.uv_heads, heads, kv_rank=self.kv_rank, rot_dim=self.rot_dim, part_o=part_o,
+                                         part_ml=part_ml, sink=self.sink_f, n_parts=launch["n_parts"])
+                else:
+                    ops.latent_heads_out(self.uv_heads, heads, kv_rank=self.kv_rank, rot_dim=self.rot_dim, mixed=mixed)
+                return ops.linear(heads.view(T, H * self.vdim), self.o_proj, out_dtype=ctx.dtype)
         else:
             ops.latent_attn_rows(qa, pages, g.block_tables, ctx.q_start, ctx.positions, ctx.ctx_len, self.sink_f,
                                  self.scale, mixed, kv_rank=self.kv_rank, rot_dim=self.rot_dim)
-        heads = torch.empty((T, H, self.vdim), dtype=ctx.dtype, device=dev)
         ops.gemm_nt_heads(mixed, self.uv_heads, heads)
         return ops.linear(heads.view(T, H * self.vdim), self.o_proj, out_dtype=ctx.dtype)

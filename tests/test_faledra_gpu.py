@@ -326,6 +326,46 @@ def test_latent_attention_sink_takes_weight_and_the_future_is_not_seen(dtype, ke
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("sizes", [(32, 16, 24), (128, 16, 40), (64, 32, 64)])
+def test_merge_and_value_projection_in_one_kernel(dtype, sizes):
+    """Steps of few rows: the partitions' results merged (with the sink) and multiplied by every
+    head's value matrix in one kernel, and the same from rows that were already merged."""
+    from lyapunov_engine_amd.kernels import ops
+
+    kv_rank, rot_dim, vdim = sizes
+    T_ctx, H, n_new, page_size = 700, 3, 2, 16
+    keys, qa, sink = latent_case(dtype, T_ctx, H, kv_rank, rot_dim, page_size, seed=vdim, n_new=n_new)
+    scale = (kv_rank + rot_dim) ** -0.5
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn(H, vdim, kv_rank, generator=g).to(tdt(dtype))
+    merged = plain_latent_attention(keys, qa, sink, scale, kv_rank)
+    if dtype == "bfloat16":
+        merged = merged.to(torch.bfloat16).double()
+    want = torch.einsum("thr,hvr->thv", merged, w.double())
+    to = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)
+    n_blocks = -(-T_ctx // page_size)
+    pages = torch.zeros(n_blocks, page_size, kv_rank + rot_dim, dtype=tdt(dtype))
+    for j in range(T_ctx):
+        pages[j // page_size, j % page_size] = keys[j]
+    for n_parts in (4, 1):
+        launch = ops.latent_attn_launch(n_new, 1, H, T_ctx, tdt(dtype), kv_rank, rot_dim, n_parts=n_parts)
+        part_o = torch.full((max(1, launch["part_o"]),), float("nan"), device=DEV)
+        part_ml = torch.full((max(1, launch["part_ml"]),), float("nan"), device=DEV)
+        mixed = torch.full((n_new, H, kv_rank), float("nan"), dtype=tdt(dtype), device=DEV)
+        ops.latent_attn(qa.to(DEV), pages.to(DEV), to([list(range(n_blocks))]), to([0, n_new]),
+                        to(np.arange(T_ctx - n_new, T_ctx)), to([T_ctx]), sink.to(DEV), scale, mixed, launch, part_o, part_ml,
+                        kv_rank=kv_rank, rot_dim=rot_dim, merge=False)
+        out = torch.empty(n_new, H, vdim, dtype=tdt(dtype), device=DEV)
+        if launch["n_parts"] > 1:
+            assert torch.isnan(mixed.float()).all(), "without the merge pass nothing writes the merged rows"
+            ops.latent_heads_out(w.to(DEV), out, kv_rank=kv_rank, rot_dim=rot_dim, part_o=part_o, part_ml=part_ml,
+                                 sink=sink.to(DEV), n_parts=launch["n_parts"])
+        else:
+            ops.latent_heads_out(w.to(DEV), out, kv_rank=kv_rank, rot_dim=rot_dim, mixed=mixed)
+        close(out, want, dtype, f"sizes {sizes}, {launch['n_parts']} partitions", floor=1e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_latent_prep_and_query_rotation(dtype):
     from lyapunov_engine_amd.kernels import ops
     from lyapunov_engine_amd.parts.rope import RotaryEncoding
