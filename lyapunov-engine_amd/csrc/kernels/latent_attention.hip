@@ -351,7 +351,7 @@ __global__ __launch_bounds__(256) void latent_combine_kernel(const float* __rest
 // workgroup per (token, head) row: the row of KV latent sums (merged from the partitions as
 // latent_combine_kernel does, or read from `mixed` when the keys were in one partition; rounded to
 // the activations' type either way, as the two-kernel path leaves it), then out[row, v] =
-// sum_r row[r] * w[head, v, r], a wave an output at a time, lanes over r.
+// sum_r row[r] * w[head, v, r], four threads an output.
 template <typename T>
 __global__ __launch_bounds__(256) void latent_heads_out_kernel(const float* __restrict__ part_o,
                                                                const float* __restrict__ part_ml,
@@ -391,14 +391,27 @@ __global__ __launch_bounds__(256) void latent_heads_out_kernel(const float* __re
     }
   }
   __syncthreads();
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, waves = blockDim.x / kWave;
+  // four neighbouring threads an output: each a quarter of the row's KV values, in pieces of four
+  // (all of a thread's loads are independent), summed across the four by two exchanges
+  using Frag = typename Mma16<T>::Frag;
+  constexpr int SEG = KV / 4;
+  const int seg = threadIdx.x % 4;
   const T* wh = w + static_cast<size_t>(head) * vdim * KV;
-  for (int v = wave; v < vdim; v += waves) {
-    const T* wr = wh + static_cast<size_t>(v) * KV;
+  for (int v0 = 0; v0 < vdim; v0 += 64) {
+    const int v = v0 + threadIdx.x / 4;
     float acc = 0.f;
-    for (int r = lane; r < KV; r += kWave) acc += rowv[r] * to_f32(wr[r]);
-    acc = wave_sum(acc);
-    if (lane == 0) out[row * vdim + v] = from_f32<T>(acc);
+    if (v < vdim) {
+      const T* wr = wh + static_cast<size_t>(v) * KV + seg * SEG;
+#pragma unroll
+      for (int r = 0; r < SEG; r += 4) {
+        const Frag f = *reinterpret_cast<const Frag*>(wr + r);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc += rowv[seg * SEG + r + e] * to_f32(f[e]);
+      }
+    }
+    acc += __shfl_xor(acc, 1, kWave);
+    acc += __shfl_xor(acc, 2, kWave);
+    if (v < vdim && seg == 0) out[row * vdim + v] = from_f32<T>(acc);
   }
 }
 
