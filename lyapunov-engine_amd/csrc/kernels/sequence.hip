@@ -237,6 +237,99 @@ __global__ void short_conv_kernel(const T* __restrict__ x, const float* __restri
   for (int k = 0; k < hist; ++k) st[static_cast<size_t>(k) * C] = from_f32<T>(input(n - hist + k));
 }
 
+// The same with 16 bytes of neighbouring channels a thread (C a multiple of the vector's length,
+// aligned operands, up to kConvTaps taps): a thread keeps its channels' taps in registers and walks
+// kConvRows rows with them (work items: groups of rows, then the requests).
+constexpr int kConvRows = 8;
+constexpr int kConvTaps = 8;
+
+template <typename T>
+__global__ void short_conv_vec_kernel(const T* __restrict__ x, const float* __restrict__ w, T* __restrict__ state,
+                                      const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions,
+                                      const int32_t* __restrict__ slots, T* __restrict__ out, int n_rows, int B, int C,
+                                      int taps, int residual) {
+  constexpr int VEC = 16 / sizeof(T);
+  typedef T VecT __attribute__((ext_vector_type(VEC)));
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
+  const int groups = (n_rows + kConvRows - 1) / kConvRows;
+  const int item = blockIdx.x;
+  const int hist = taps - 1;
+  if (c >= C) return;
+  auto load = [&](const T* p) { return *reinterpret_cast<const VecT*>(p); };
+  auto store = [&](T* p, const float (&v)[VEC]) {
+    VecT o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o[e] = from_f32<T>(v[e]);
+    *reinterpret_cast<VecT*>(p) = o;
+  };
+  float wr[VEC][kConvTaps];   // this thread's channels x taps
+#pragma unroll
+  for (int e = 0; e < VEC; ++e)
+#pragma unroll
+    for (int j = 0; j < kConvTaps; ++j) wr[e][j] = j < taps ? w[static_cast<size_t>(c + e) * taps + j] : 0.f;
+  if (item < groups) {
+    const int live = q_start[B];
+    for (int row = item * kConvRows; row < min(n_rows, (item + 1) * kConvRows); ++row) {
+      float acc[VEC];
+      if (row >= live) {   // rows past the last request belong to nobody
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+        store(out + static_cast<size_t>(row) * C + c, acc);
+        continue;
+      }
+      const int b = owner_of(q_start, B, row);
+      if (row - q_start[b] < hist) continue;   // the request's item does the rows that read its slot
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+#pragma unroll
+      for (int j = 0; j < kConvTaps; ++j) {
+        if (j < taps) {
+          const VecT v = load(x + static_cast<size_t>(row - hist + j) * C + c);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            acc[e] += wr[e][j] * to_f32(v[e]);
+            if (residual && j == hist) acc[e] += to_f32(v[e]);
+          }
+        }
+      }
+      store(out + static_cast<size_t>(row) * C + c, acc);
+    }
+    return;
+  }
+  const int b = item - groups;
+  const int q0 = q_start[b], n = q_start[b + 1] - q0;
+  if (n <= 0) return;
+  const bool fresh = positions[q0] == 0;
+  T* st = hist > 0 ? state + (static_cast<size_t>(slots[b]) * hist) * C + c : nullptr;
+  auto input = [&](int idx) -> VecT {   // input at local index idx (negative: from the slot)
+    if (idx >= 0) return load(x + static_cast<size_t>(q0 + idx) * C + c);
+    VecT z;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) z[e] = from_f32<T>(0.f);
+    return fresh ? z : load(st + static_cast<size_t>(idx + hist) * C);
+  };
+  const int head = n < hist ? n : hist;
+  for (int i = 0; i < head; ++i) {
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+#pragma unroll
+    for (int j = 0; j < kConvTaps; ++j) {
+      if (j < taps) {
+        const VecT v = input(i - hist + j);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          acc[e] += wr[e][j] * to_f32(v[e]);
+          if (residual && j == hist) acc[e] += to_f32(v[e]);
+        }
+      }
+    }
+    store(out + static_cast<size_t>(q0 + i) * C + c, acc);
+  }
+  // slot entry k becomes the input at local index n - hist + k (rising k reads entries k + n > k only)
+  for (int k = 0; k < hist; ++k) *reinterpret_cast<VecT*>(st + static_cast<size_t>(k) * C) = input(n - hist + k);
+}
+
 // ------------------------------------------------------------- activations
 __device__ __forceinline__ float softplus_f(float v) { return v > 20.f ? v : log1pf(expf(v)); }
 
@@ -322,7 +415,7 @@ __global__ void mingru_scan_kernel(const float* __restrict__ pre, const float* _
 //   outputs:   a chunk folds the summaries of the chunks before it into its incoming state, walks
 //              its rows again and writes them; a request's last chunk writes the state slot.
 // Chunk c of the launch maps to (request, chunk of the request) by a walk over q_start.
-constexpr int kScanChunk = 64;
+constexpr int kScanChunk = 32;
 
 __device__ __forceinline__ bool scan_chunk_of(const int32_t* __restrict__ q_start, int B, int item, int& b, int& first,
                                               int& r0, int& r1) {
@@ -355,6 +448,7 @@ __global__ void mingru_chunk_summary_kernel(const float* __restrict__ pre, const
     init[static_cast<size_t>(b) * W + c] = positions[r0] == 0 ? 0.f : state[static_cast<size_t>(slots[b]) * W + c];
   const float zb = bz[c], xb = bx[c];
   float P = 1.f, S = 0.f;
+#pragma unroll 8
   for (int t = r0; t < r1; ++t) {
     const float* row = pre + static_cast<size_t>(t) * 3 * W;
     const float z = sigmoid_f(row[c] + zb);
@@ -380,6 +474,7 @@ __global__ void mingru_chunk_output_kernel(const float* __restrict__ pre, const 
   for (int k = first; k < static_cast<int>(blockIdx.x); ++k)
     S = prod[static_cast<size_t>(k) * W + c] * S + end[static_cast<size_t>(k) * W + c];
   const float zb = bz[c], xb = bx[c];
+#pragma unroll 8
   for (int t = r0; t < r1; ++t) {
     const float* row = pre + static_cast<size_t>(t) * 3 * W;
     const float z = sigmoid_f(row[c] + zb);
@@ -636,6 +731,24 @@ int lyp_short_conv(const void* x, const float* w, void* state, const int32_t* q_
   LYP_REQUIRE(taps == 1 || state != nullptr, "short_conv: %d taps need a state", taps);
   LYP_REQUIRE(x != out, "short_conv: in place is not possible");
   if (n_rows == 0) return 0;
+  const int vlen = dtype == kF32 ? 4 : 8;
+  auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if ((dtype == kF32 || dtype == kBF16) && C % vlen == 0 && taps <= kConvTaps && aligned(x) && aligned(out) &&
+      aligned(state)) {
+    const int units = C / vlen;
+    const int vt = units >= 256 ? 256 : 64 * ((units + 63) / 64);
+    dim3 vgrid((n_rows + kConvRows - 1) / kConvRows + B, (units + vt - 1) / vt);
+    if (dtype == kF32)
+      short_conv_vec_kernel<float><<<vgrid, vt, 0, stream>>>(static_cast<const float*>(x), w,
+                                                             static_cast<float*>(state), q_start, positions, slots,
+                                                             static_cast<float*>(out), n_rows, B, C, taps, residual);
+    else
+      short_conv_vec_kernel<bf16_t><<<vgrid, vt, 0, stream>>>(static_cast<const bf16_t*>(x), w,
+                                                              static_cast<bf16_t*>(state), q_start, positions, slots,
+                                                              static_cast<bf16_t*>(out), n_rows, B, C, taps, residual);
+    LYP_LAUNCH_CHECK("short_conv");
+    return 0;
+  }
   const int threads = C >= 256 ? 256 : 64 * ((C + 63) / 64);
   dim3 grid(n_rows + B, (C + threads - 1) / threads);
   if (dtype == kF32)
@@ -693,7 +806,7 @@ int lyp_mingru_scan(const float* pre, const float* bz, const float* bx, float* s
 }
 
 // The recurrence in chunks (see mingru_chunk_summary_kernel): n_rows rows of B requests; ws holds
-// (2 * (n_rows / 64 rounded up + B) + B) * W floats.
+// (2 * (n_rows / 32 rounded up + B) + B) * W floats.
 int lyp_mingru_scan_chunks(const float* pre, const float* bz, const float* bx, float* state, const int32_t* q_start,
                            const int32_t* positions, const int32_t* slots, void* out, int out_dtype, int n_rows, int B,
                            int W, float* ws, long long ws_floats, hipStream_t stream) {

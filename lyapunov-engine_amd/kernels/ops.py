@@ -954,7 +954,7 @@ def mingru_scan(pre: torch.Tensor, bz: torch.Tensor, bx: torch.Tensor, state: to
     """The minGRU recurrence over the step's rows, request by request: pre float [T, 3 W] holds the
     update-gate, candidate and output-gate projections side by side; state float [slots, W].
     Without a workspace a thread walks all rows of its request and channel (steps of few rows per
-    request); with one (``mingru_scan_workspace`` floats) the rows go in chunks of 64 that run side by
+    request); with one (``mingru_scan_workspace`` floats) the rows go in chunks of 32 that run side by
     side: a pass for every chunk's summary, a pass for the outputs (the recurrence is linear in the state)."""
     _dev(pre, bz, bx, state, q_start, positions, slots, out)
     _f32(pre, bz, bx, state)
@@ -978,8 +978,8 @@ def mingru_scan(pre: torch.Tensor, bz: torch.Tensor, bx: torch.Tensor, state: to
 
 
 def mingru_scan_workspace(T: int, B: int, W: int) -> int:
-    """Floats of the workspace with which ``mingru_scan`` walks a step's rows in chunks of 64."""
-    return (2 * (-(-T // 64) + B) + B) * W
+    """Floats of the workspace with which ``mingru_scan`` walks a step's rows in chunks of 32."""
+    return (2 * (-(-T // 32) + B) + B) * W
 
 
 def latent_prep(d: torch.Tensor, wq: torch.Tensor, wkv: torch.Tensor, positions: torch.Tensor,

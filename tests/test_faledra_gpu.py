@@ -79,14 +79,14 @@ def test_branch_join_and_following_norm(dtype, H):
     close(hd, h.double() + shift.double(), "float32", "shift alone")
 
 
+@pytest.mark.parametrize("C", [70, 72])      # one channel a thread, and 16 bytes of channels a thread
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("taps", [1, 2, 3, 5])
-def test_short_conv_in_portions_with_slots_used_again(dtype, taps):
+def test_short_conv_in_portions_with_slots_used_again(dtype, taps, C):
     """Three requests in portions of every size (shorter than the filter's memory too), beside each
     other and in slots another request used before, against the whole sequences."""
     from lyapunov_engine_amd.kernels import ops
 
-    C = 70
     g = torch.Generator().manual_seed(taps)
     w = torch.randn(C, taps, generator=g)
     seqs = {r: torch.randn(n, C, generator=g).to(tdt(dtype)) for r, n in (("a", 23), ("b", 9), ("c", 14))}
