@@ -76,7 +76,8 @@ def run_generate(args) -> int:
 
 def build_parser() -> argparse.ArgumentParser:
     parser = argparse.ArgumentParser(prog="lyapunov",
-                                     description="Lyapunov Engine for AMD MI355X: Llama inference on one GPU")
+                                     description="Lyapunov Engine for AMD MI355X: decoder inference on one GPU (the architecture is the "
+                                                 "one the model folder's config.json names)")
     sub = parser.add_subparsers(dest="subcommand", required=True)
     gen = sub.add_parser("generate", help="Run text generation from prompt")
     gen.add_argument("--model", type=str, required=True, help="local model directory (config.json, *.safetensors)")

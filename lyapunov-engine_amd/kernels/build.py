@@ -47,7 +47,8 @@ RUNTIME_SOURCES = ["runtime/cache_manager.cpp", "runtime/scheduler.cpp", "runtim
 # to 256 is compiled when a model first asks for it.
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
 # (latent, rotated part) sizes of the latent attention library compiled ahead of time; others on first use.
-PREBUILT_LATENT_SIZES = ((64, 32), (96, 16), (64, 16), (256, 32))
+PREBUILT_LATENT_SIZES = ((16, 0), (16, 16), (16, 32), (32, 0), (32, 16), (32, 48), (48, 0), (48, 16), (64, 16), (64, 32),
+                         (64, 64), (96, 16), (128, 16), (128, 32), (256, 32), (512, 32))
 
 _lock = threading.Lock()
 

@@ -49,7 +49,7 @@ CONFIGS = {
                 taps=1, mult=1.0, emb_scale=1.0, eps=1e-6),
     "C": config(320, 128, [latent(4, 32, 32, 16, 64, 64, ff=192),
                            gru(96, ff=64),
-                           latent(8, 16, 16, 32, 48, 96, base=50000.0)],
+                           latent(8, 16, 16, 32, 48, 96, base=20000.0)],
                 taps=2, loop=(0, 2, 1), mult=0.8, emb_scale=8.0, eps=1e-6),
 }
 BLOCK_SIZE = {"A": 4, "B": 16, "C": 16}
