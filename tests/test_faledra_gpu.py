@@ -571,6 +571,30 @@ def test_the_given_shape_of_things_is_not_assumed(tmp_path, dtype):
     compare(t, got, plain_logits(folder, t.requests), dtype, "one of everything", tol=None if dtype == "float32" else TOL16)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("layers", ["recurrent only", "no rotated part", "attention only, looped four times"])
+def test_other_orders_of_layers(tmp_path, dtype, layers):
+    """Models without any paged cache (recurrent layers alone), with heads that have no rotated
+    part, and of attention layers alone in a loop: portions, then single tokens, two requests."""
+    if layers == "recurrent only":
+        cfg = config(111, 40, [gru(24, ff=56), gru(40)], taps=3, loop=(1, 2, 2), mult=0.9)
+    elif layers == "no rotated part":
+        cfg = config(111, 48, [latent(2, 16, 0, 16, 24, 32, ff=64), gru(32, ff=40)], taps=2)
+    else:
+        cfg = config(111, 64, [latent(4, 16, 16, 16, 32, 48, ff=96), latent(2, 32, 16, 24, 40, 64)], taps=5,
+                     loop=(0, 2, 4), mult=0.5)
+    folder = write_model(str(tmp_path / "m"), cfg, seed=9, dtype=dtype)
+    reqs = {"x": random_tokens(50, 111, seed=1), "y": random_tokens(21, 111, seed=2)}
+    t = Trace(reqs)
+    t.step([("x", 30)])
+    t.step([("x", 3), ("y", 19)])
+    for _ in range(2):
+        t.step([("x", 1), ("y", 1)])
+    t.step([("x", 15)], end=["x", "y"])
+    got = replay(folder, dtype, t, block_size=8)
+    compare(t, got, plain_logits(folder, t.requests), dtype, layers, tol=None if dtype == "float32" else TOL16)
+
+
 # ------------------------------------------------------------------- generation
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "C"])
