@@ -31,6 +31,7 @@ class GroupConfig:
     num_pages: int
     page_size: int = 16
     window: int = 0
+    keep_first: int = 0    # with a window: the pages of a request's first keep_first tokens are never given back
 
 
 class CacheManager:
@@ -41,7 +42,8 @@ class CacheManager:
         arr = lambda vals: (c_int * n)(*vals)
         self._h = self._lib.lyp_cache_create(n, arr([g.num_pages for g in self.groups]),
                                              arr([g.page_size for g in self.groups]),
-                                             arr([g.window for g in self.groups]), num_state_slots)
+                                             arr([g.window for g in self.groups]),
+                                             arr([g.keep_first for g in self.groups]), num_state_slots)
         if not self._h:
             raise CacheError(runtime_lib.last_error())
         self.num_state_slots = num_state_slots

@@ -25,7 +25,7 @@ def lib() -> ctypes.CDLL:
     i32p, i64p = POINTER(c_int32), POINTER(c_int64)
     L.lyp_rt_last_error.restype = c_char_p
     L.lyp_cache_create.restype = c_void_p
-    L.lyp_cache_create.argtypes = [c_int, POINTER(c_int), POINTER(c_int), POINTER(c_int), c_int]
+    L.lyp_cache_create.argtypes = [c_int, POINTER(c_int), POINTER(c_int), POINTER(c_int), POINTER(c_int), c_int]
     L.lyp_cache_destroy.argtypes = [c_void_p]
     for name in ("add", "has", "length", "capacity", "free", "state_slot", "max_length"):
         getattr(L, f"lyp_cache_{name}").argtypes = [c_void_p, c_int64]

@@ -63,13 +63,16 @@ class LayerCall:
     ``writes``  false: the mixer only reads the buffer (another call filled it)
                 and computes no keys and values of its own;
     ``shift``   a row of the model's stream shift (``ModelSpec.stream_shift``)
-                that is added to the residual stream right before this call.
+                that is added to the residual stream right before this call;
+    ``reinject`` true: the embedding's output (the stream's first value, row by
+                row) is added to the residual stream right before this call.
     """
 
     layer: int
     cache: int
     writes: bool = True
     shift: Optional[int] = None
+    reinject: bool = False
 
 
 @dataclass(frozen=True)

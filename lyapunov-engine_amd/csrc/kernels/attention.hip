@@ -73,6 +73,7 @@ struct PagedKV {
   const int32_t* table;  // this request's row of the block table
   int nkv, bs, kvh;
   int max_blocks;        // width of the row: an index below it may always be read
+  int keep = 0;          // keys below this are wanted although they lie before `lo` (a window that keeps the first tokens)
 };
 
 // The table entry for a key, read whether or not the key is inside the
@@ -88,7 +89,7 @@ template <typename T>
 __device__ __forceinline__ void load_k_page(Frag<T> (&kf)[kSteps], const PagedKV& kv, int kb0, int lo, int hi,
                                             int lane, int page) {
   const int key = kb0 + lane % 16;
-  if (key >= lo && key < hi) {
+  if ((key >= lo || key < kv.keep) && key < hi) {
     if (page >= 0) {
       const T* row = static_cast<const T*>(kv.kpool) +
                      ((static_cast<size_t>(page) * kv.nkv + kv.kvh) * kv.bs + key % kv.bs) * HD +
@@ -123,7 +124,7 @@ __device__ __forceinline__ void load_v_page(Frag<T> (&vf)[kSteps], const PagedKV
 #pragma unroll
   for (int db = 0; db < kSteps; ++db) vf[db] = zero_frag<T>();
   if (kv.bs % 4 == 0) {
-    if (key0 < hi && key0 + 3 >= lo) {
+    if (key0 < hi && (key0 + 3 >= lo || key0 < kv.keep)) {
       const int page = page0;
       if (page >= 0) {
         const T* base = vpool + (static_cast<size_t>(page) * kv.nkv + kv.kvh) * HD * kv.bs + key0 % kv.bs;
@@ -132,7 +133,7 @@ __device__ __forceinline__ void load_v_page(Frag<T> (&vf)[kSteps], const PagedKV
           Frag<T> f = *reinterpret_cast<const Frag<T>*>(base + static_cast<size_t>(db * 16 + r) * kv.bs);
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            if (key0 + i < lo || key0 + i >= hi) f[i] = from_f32<T>(0.f);
+            if ((key0 + i < lo && key0 + i >= kv.keep) || key0 + i >= hi) f[i] = from_f32<T>(0.f);
           vf[db] = f;
         }
       }
@@ -141,7 +142,7 @@ __device__ __forceinline__ void load_v_page(Frag<T> (&vf)[kSteps], const PagedKV
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = key0 + i;
-      if (key < lo || key >= hi) continue;
+      if ((key < lo && key >= kv.keep) || key >= hi) continue;
       const int page = kv.table[key / kv.bs];
       if (page < 0) continue;
       const T* base = vpool + (static_cast<size_t>(page) * kv.nkv + kv.kvh) * HD * kv.bs + key % kv.bs;
@@ -207,12 +208,12 @@ __device__ __forceinline__ float lane_groups_max(float m) {
 // operands of the P.V products: one maximum, one rescaling and one pass of
 // exponentials for all of them, which is most of the arithmetic outside the
 // matrix cores.  `pos` is the column's absolute position; a key is visible when
-// key <= pos, key < hi and (window == 0 or key > pos - window).  With MASKED
+// key <= pos, key < hi and (window == 0 or key > pos - window or key < keep).  With MASKED
 // false every key is visible to every column and the tests are skipped.
 template <typename T, bool MASKED, int NB>
 __device__ __forceinline__ void softmax_group(const f32x4 (&s)[NB], Frag<T> (&pf)[NB], float scale_log2, int kb0,
-                                              int pos, int window, int hi, Softmax& st, f32x4 (&o)[kSteps],
-                                              int lane) {
+                                              int pos, int window, int keep, int hi, Softmax& st,
+                                              f32x4 (&o)[kSteps], int lane) {
   float sv[NB][4];
   float mx = LYP_NEG_INF;
 #pragma unroll
@@ -221,7 +222,7 @@ __device__ __forceinline__ void softmax_group(const f32x4 (&s)[NB], Frag<T> (&pf
     for (int i = 0; i < 4; ++i) {
       if constexpr (MASKED) {
         const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
-        const bool vis = key <= pos && key < hi && (window == 0 || key > pos - window);
+        const bool vis = key <= pos && key < hi && (window == 0 || key > pos - window || key < keep);
         sv[u][i] = vis ? s[u][i] * scale_log2 : LYP_NEG_INF;
       } else {
         sv[u][i] = s[u][i] * scale_log2;
@@ -255,6 +256,18 @@ __device__ __forceinline__ float lane_groups_sum(float v) {
   return v;
 }
 
+// What an accumulated output (relative to the maximum m, base-2 domain) is multiplied by at the
+// end: 1 / l, or with a sink, a score without key or value that stands in the denominator once,
+// 2^(m - M) / (l 2^(m - M) + 2^(sink - M)) with M the larger of m and the sink.  0 when no key
+// was seen.
+__device__ __forceinline__ float final_scale(float m, float l, const float* sink, int head) {
+  if (sink == nullptr) return l > 0.f ? 1.0f / l : 0.f;
+  const float s2 = sink[head] * kLog2e;
+  const float big = fmaxf(m, s2);
+  const float a = fast_exp2(m - big);   // 0 when nothing was seen (m = -inf)
+  return a / (l * a + fast_exp2(s2 - big));
+}
+
 // --------------------------------------------------------------------- prefill
 // grid (tiles * sub-tiles, nkv * head_groups); 256 threads (four waves).  A
 // workgroup takes QW consecutive new tokens of one request and GH query heads of
@@ -281,7 +294,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int n_tiles, int nh, int nkv,
-    int bs, int window, float scale_log2) {
+    int bs, int window, float scale_log2, int keep, const float* __restrict__ sink) {
   using PT = PrefillTile<T>;
   constexpr int KT = PT::kKeys, NB = KT / 16, VEC = PT::kVec;
   constexpr int QW = (4 / GH) * QB * 16;  // new tokens per workgroup
@@ -394,7 +407,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       if (tid + n * 256 >= PT::kKVecs) continue;
       {  // keys: 16 bytes of key kt0 + k_row
         const int key = kt0 + k_row[n];
-        if (key >= lo_wg && key < hi_wg) {
+        if ((key >= lo_wg || key < keep) && key < hi_wg) {
           const int page = table[key / bs];
           if (page >= 0)
             kreg[n] = *reinterpret_cast<const VecT*>(
@@ -403,7 +416,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       }
       {  // values: 16-key blocks one after the other, inside a block dimension by dimension
         const int d = v_d[n], key0 = kt0 + 16 * v_blk[n] + v_c[n];
-        if (key0 < hi_wg && key0 + VEC > lo_wg) {
+        if (key0 < hi_wg && (key0 + VEC > lo_wg || key0 < keep)) {
           if (v_vectors) {
             const int page = table[key0 / bs];
             if (page >= 0) {
@@ -411,14 +424,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                   vp + ((static_cast<size_t>(page) * nkv + kvh) * HD + d) * bs + key0 % bs);
 #pragma unroll
               for (int e = 0; e < VEC; ++e)
-                if (key0 + e < lo_wg || key0 + e >= hi_wg) x[e] = from_f32<T>(0.f);
+                if ((key0 + e < lo_wg && key0 + e >= keep) || key0 + e >= hi_wg) x[e] = from_f32<T>(0.f);
               vreg[n] = x;
             }
           } else {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
               const int key = key0 + e;
-              if (key < lo_wg || key >= hi_wg) continue;
+              if ((key < lo_wg && key >= keep) || key >= hi_wg) continue;
               const int page = table[key / bs];
               if (page >= 0) vreg[n][e] = vp[((static_cast<size_t>(page) * nkv + kvh) * HD + d) * bs + key % bs];
             }
@@ -480,10 +493,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       const bool full = kt0 + KT - 1 <= pos0[b] && kt0 >= lo_wg && pos0[b] + 15 <= pos_last_wg &&
                         (window == 0 || kt0 > pos0[b] + 15 - window);
       if (full)
-        softmax_group<T, false, NB>(sc[b], pf[b], scale_log2, kt0, pos0[b] + col, window, hi_wg, st[b], o[b], lane);
+        softmax_group<T, false, NB>(sc[b], pf[b], scale_log2, kt0, pos0[b] + col, window, keep, hi_wg, st[b], o[b],
+                                    lane);
       else
-        softmax_group<T, true, NB>(sc[b], pf[b], scale_log2, kt0, col_valid[b] ? pos0[b] + col : -1, window, hi_wg,
-                                   st[b], o[b], lane);
+        softmax_group<T, true, NB>(sc[b], pf[b], scale_log2, kt0, col_valid[b] ? pos0[b] + col : -1, window, keep,
+                                   hi_wg, st[b], o[b], lane);
     }
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
@@ -498,19 +512,25 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     }
   };
 
-  const int kt_first = (lo_wg / KT) * KT;
+  // The tiles in the order they are walked: those that hold kept first tokens the window no
+  // longer covers, then the window's.
+  const int kt_window = (lo_wg / KT) * KT;
+  const int kept_end = min((keep + KT - 1) / KT * KT, kt_window);   // 0 without a window or kept tokens
+  const int kt_first = kept_end > 0 ? 0 : kt_window;
+  auto tile_after = [&](int kt0) { return kt0 + KT < kept_end ? kt0 + KT : max(kt0 + KT, kt_window); };
   int pages[NB];
   tile_pages(kt_first, pages);
   fetch(kt_first, pages);
-  tile_pages(kt_first + KT, pages);
+  tile_pages(tile_after(kt_first), pages);
   stash(0);
   __syncthreads();
   int buf = 0;
-  for (int kt0 = kt_first; kt0 < hi_wg; kt0 += KT) {
-    const bool more = kt0 + KT < hi_wg;
+  for (int kt0 = kt_first, kt_next; kt0 < hi_wg; kt0 = kt_next) {
+    kt_next = tile_after(kt0);
+    const bool more = kt_next < hi_wg;
     if (more) {
-      fetch(kt0 + KT, pages);
-      tile_pages(kt0 + 2 * KT, pages);  // for the fetch of the next round
+      fetch(kt_next, pages);
+      tile_pages(tile_after(kt_next), pages);  // for the fetch of the next round
     }
     if (wave_active && kt0 <= pos_last_w) compute(buf, kt0);
     if (PT::kBufs == 1) __syncthreads();  // everyone is done with the only buffer before it is overwritten
@@ -524,7 +544,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   for (int b = 0; b < QB; ++b) {
     const float l = lane_groups_sum(st[b].lsum);
     if (!col_valid[b]) continue;
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const float inv = final_scale(st[b].m, l, sink, head);
     const size_t token = static_cast<size_t>(tok0) + q0_w + 16 * b + col;
     T* orow = out + token * out_stride + static_cast<size_t>(head) * HD + 4 * (lane / 16);
 #pragma unroll
@@ -634,7 +654,8 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
     const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int n_tiles, int nh, int nkv,
-    int bs, int window, float scale_log2, int paired, float* __restrict__ part_o, float* __restrict__ part_ml,
+    int bs, int window, float scale_log2, const float* __restrict__ sink, int paired, float* __restrict__ part_o,
+    float* __restrict__ part_ml,
     int n_parts) {
   using T = bf16_t;
   using WT = WideTile;
@@ -919,7 +940,7 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
         }
       }
     } else if (col_valid && set == 0) {
-      const float inv = lacc[0] > 0.f ? 1.0f / lacc[0] : 0.f;
+      const float inv = final_scale(m_run, lacc[0], sink, head);
       T* orow = out + (static_cast<size_t>(tok0) + q0_w + col) * out_stride + static_cast<size_t>(head) * HD + 4 * grp;
 #pragma unroll
       for (int db = 0; db < kSteps; ++db) {
@@ -937,7 +958,7 @@ template <typename T>
 __global__ __launch_bounds__(64) void attn_merge_parts_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int n_parts,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0,
-    T* __restrict__ out, int out_stride, int nh) {
+    T* __restrict__ out, int out_stride, int nh, const float* __restrict__ sink) {
   const int head = blockIdx.x, in_tile = blockIdx.y, tile = blockIdx.z, lane = threadIdx.x;
   const int seq = tile_seq[tile];
   const int tok0 = q_start[seq], q_len = q_start[seq + 1] - tok0;
@@ -950,7 +971,7 @@ __global__ __launch_bounds__(64) void attn_merge_parts_kernel(
   const float m_safe = m == LYP_NEG_INF ? 0.f : m;
   float l = 0.f;
   for (int p = 0; p < n_parts; ++p) l += fast_exp2(ml[p].x - m_safe) * ml[p].y;
-  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  const float inv = final_scale(m, l, sink, head);
   T* orow = out + (static_cast<size_t>(tok0) + q) * out_stride + static_cast<size_t>(head) * HD;
   for (int d = lane; d < HD; d += kWave) {
     float acc = 0.f;
@@ -1001,7 +1022,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ dec_seqs,
     float* __restrict__ part_o, float* __restrict__ part_ml, int max_parts, int most_keys_per_wave, int nh, int nkv,
-    int bs, int window, float scale_log2, T* __restrict__ out, int out_stride) {
+    int bs, int window, float scale_log2, T* __restrict__ out, int out_stride, int keep,
+    const float* __restrict__ sink) {
   extern __shared__ float s_decode[];
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // the same in every lane: keeps what follows scalar
@@ -1032,7 +1054,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   const int pos = ctx - 1;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   // (A request without keys still gets its row of zeros written when no combine pass follows.)
-  if (!WHOLE && (part * block_keys >= ctx || (part + 1) * block_keys <= lo)) return;  // the whole workgroup
+  if (!WHOLE && (part * block_keys >= ctx || ((part + 1) * block_keys <= lo && part * block_keys >= keep)))
+    return;  // the whole workgroup
 
   const int col = lane % 16;
   const bool col_valid = h0 + col < g;
@@ -1046,9 +1069,12 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   for (int db = 0; db < kSteps; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
   Softmax st{LYP_NEG_INF, 0.f};
 
-  PagedKV kv{kpool, vpool, table, nkv, bs, kvh, max_blocks};
+  PagedKV kv{kpool, vpool, table, nkv, bs, kvh, max_blocks, keep};
   const bool aligned = bs % 16 == 0;
-  const int k_first = max(k_begin, (lo / 16) * 16);
+  // This wave's groups of keys in the order they are walked: those that hold kept first tokens
+  // the window no longer covers, then the window's.
+  const int k_window = max(k_begin, (lo / 16) * 16);
+  const int k_first = k_begin < keep ? k_begin : k_window;
   const int k_end = min(ctx, k_begin + keys_per_wave);
 
   Frag<T> kf[kDecodeDepth][kSteps], vf[kDecodeDepth][kSteps];
@@ -1097,8 +1123,10 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     load_k_of(u, k_first + 16 * u);
     load_v_of(u, k_first + 16 * u);
   }
-  for (int kb0 = k_first; kb0 < k_end; kb0 += GK) {
-    const bool more = kb0 + GK < k_end;
+  auto group_after = [&](int kb0) { return kb0 + GK < keep ? kb0 + GK : max(kb0 + GK, k_window); };
+  for (int kb0 = k_first, kb_next; kb0 < k_end; kb0 = kb_next) {
+    kb_next = group_after(kb0);
+    const bool more = kb_next < k_end;
     f32x4 s[kDecodeDepth];
 #pragma unroll
     for (int u = 0; u < kDecodeDepth; ++u) {
@@ -1107,22 +1135,23 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
       for (int k = 0; k < kSteps; ++k) s[u] = Mma16<T>::mma(kf[u][k], qf[k], s[u]);
     }
     if (more) {
-      pages_of(kb0 + GK);  // the values of the next group, asked for below, lie in the same pages
+      pages_of(kb_next);  // the values of the next group, asked for below, lie in the same pages
 #pragma unroll
-      for (int u = 0; u < kDecodeDepth; ++u) load_k_of(u, kb0 + GK + 16 * u);
+      for (int u = 0; u < kDecodeDepth; ++u) load_k_of(u, kb_next + 16 * u);
     }
     Frag<T> pf[kDecodeDepth];
     if (aligned && kb0 >= lo && kb0 + GK <= k_end)
-      softmax_group<T, false, kDecodeDepth>(s, pf, scale_log2, kb0, pos, window, k_end, st, o, lane);
+      softmax_group<T, false, kDecodeDepth>(s, pf, scale_log2, kb0, pos, window, keep, k_end, st, o, lane);
     else
-      softmax_group<T, true, kDecodeDepth>(s, pf, scale_log2, kb0, col_valid ? pos : -1, window, k_end, st, o, lane);
+      softmax_group<T, true, kDecodeDepth>(s, pf, scale_log2, kb0, col_valid ? pos : -1, window, keep, k_end, st, o,
+                                           lane);
 #pragma unroll
     for (int u = 0; u < kDecodeDepth; ++u)
 #pragma unroll
       for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[u][db], pf[u], o[db]);
     if (more) {
 #pragma unroll
-      for (int u = 0; u < kDecodeDepth; ++u) load_v_of(u, kb0 + GK + 16 * u);
+      for (int u = 0; u < kDecodeDepth; ++u) load_v_of(u, kb_next + 16 * u);
     }
   }
 
@@ -1156,7 +1185,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     }
     if constexpr (WHOLE) {
       out[token * out_stride + static_cast<size_t>(kvh * g + h0 + c) * HD + d] =
-          from_f32<T>(lsum > 0.f ? acc / lsum : 0.f);
+          from_f32<T>(acc * final_scale(m, lsum, sink, kvh * g + h0 + c));
     } else {
       const size_t pidx = (static_cast<size_t>(slot) * nh + kvh * g + h0 + c) * max_parts + part;
       part_o[pidx * HD + d] = acc;
@@ -1175,7 +1204,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int max_parts,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ dec_seqs, T* __restrict__ out, int out_stride, int nh, int window,
-    int most_block_keys) {
+    int most_block_keys, int keep, const float* __restrict__ sink) {
   const int head = blockIdx.x, slot = blockIdx.y, lane = threadIdx.x;
   const int seq = dec_seqs ? dec_seqs[slot] : slot;
   const size_t base = (static_cast<size_t>(slot) * nh + head) * max_parts;
@@ -1203,14 +1232,20 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
   }
   const int block_keys = kDecodeWaves * decode_keys_per_wave(ctx, most_block_keys / kDecodeWaves);
   const int lo = window > 0 ? max(0, ctx - window) : 0;
-  const int p_lo = lo / block_keys;
   const int p_hi = (ctx + block_keys - 1) / block_keys;
+  // partitions [p_lo, p_hi) hold keys; with kept first tokens that the window no longer covers
+  // these are walked from partition 0 and the ones in between dropped (`live`)
+  const int p_win = lo / block_keys;
+  const int p_keep = window > 0 ? (min(keep, lo) + block_keys - 1) / block_keys : 0;
+  const int p_lo = p_keep > 0 ? 0 : p_win;
+  auto live = [&](int p) { return p < p_hi && (p >= p_win || p < p_keep); };
 
   float m = LYP_NEG_INF;
 #pragma unroll
   for (int p = 0; p < kFirst; ++p)
-    if (p >= p_lo && p < p_hi) m = fmaxf(m, ml_first[p].x);
-  for (int p = max(p_lo, kFirst) + lane; p < p_hi; p += kWave) m = fmaxf(m, ml[p].x);
+    if (live(p)) m = fmaxf(m, ml_first[p].x);
+  for (int p = max(p_lo, kFirst) + lane; p < p_hi; p += kWave)
+    if (live(p)) m = fmaxf(m, ml[p].x);
   m = wave_max(m);
   const float m_safe = m == LYP_NEG_INF ? 0.f : m;
   // every lane adds up the same terms in the same order: partitions 0 .. kFirst - 1, then the rest by lanes
@@ -1218,13 +1253,14 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
   float w_first[kFirst];
 #pragma unroll
   for (int p = 0; p < kFirst; ++p) {
-    w_first[p] = (p >= p_lo && p < p_hi) ? fast_exp2(ml_first[p].x - m_safe) : 0.f;
-    l += (p >= p_lo && p < p_hi) ? w_first[p] * ml_first[p].y : 0.f;
+    w_first[p] = live(p) ? fast_exp2(ml_first[p].x - m_safe) : 0.f;
+    l += live(p) ? w_first[p] * ml_first[p].y : 0.f;
   }
   float l_rest = 0.f;
-  for (int p = max(p_lo, kFirst) + lane; p < p_hi; p += kWave) l_rest += fast_exp2(ml[p].x - m_safe) * ml[p].y;
+  for (int p = max(p_lo, kFirst) + lane; p < p_hi; p += kWave)
+    if (live(p)) l_rest += fast_exp2(ml[p].x - m_safe) * ml[p].y;
   l += wave_sum(l_rest);
-  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  const float inv = final_scale(m, l, sink, head);
 
   T* orow = out + static_cast<size_t>(tok) * out_stride + static_cast<size_t>(head) * HD;
 #pragma unroll
@@ -1233,15 +1269,17 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
     if (d >= HD) continue;
     float acc = 0.f;
 #pragma unroll
-    for (int p = 0; p < kFirst; ++p) acc += (p >= p_lo && p < p_hi) ? w_first[p] * o_first[k][p] : 0.f;
+    for (int p = 0; p < kFirst; ++p) acc += live(p) ? w_first[p] * o_first[k][p] : 0.f;
 #pragma unroll 4
-    for (int p = max(p_lo, kFirst); p < p_hi; ++p) acc += fast_exp2(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
+    for (int p = max(p_lo, kFirst); p < p_hi; ++p)
+      if (live(p)) acc += fast_exp2(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
     orow[d] = from_f32<T>(acc * inv);
   }
   if constexpr (HD < kWave || HD % kWave != 0) {   // head sizes that are no multiple of 64: the dimensions past the lanes' share
     for (int d = lane + kWave * kPerLane; d < HD; d += kWave) {
       float acc = 0.f;
-      for (int p = p_lo; p < p_hi; ++p) acc += fast_exp2(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
+      for (int p = p_lo; p < p_hi; ++p)
+        if (live(p)) acc += fast_exp2(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
       orow[d] = from_f32<T>(acc * inv);
     }
   }
@@ -1321,9 +1359,11 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
                      const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
                      const int32_t* q_start, const int32_t* ctx_len, const int32_t* tile_seq,
                      const int32_t* tile_q0, int n_tiles, int nh, int nkv, int bs, int window, float scale,
-                     int pair, float* part_o, float* part_ml, int n_parts, hipStream_t stream) {
+                     int pair, float* part_o, float* part_ml, int n_parts, int keep_first, const float* sink,
+                     hipStream_t stream) {
   if (check_common("attn_prefill", nh, nkv, bs, max_blocks, q_stride, out_stride, window)) return -1;
-  LYP_REQUIRE(n_tiles >= 0, "attn_prefill: %d tiles", n_tiles);
+  LYP_REQUIRE(n_tiles >= 0 && keep_first >= 0, "attn_prefill: %d tiles, %d kept first tokens", n_tiles, keep_first);
+  const int keep = window > 0 ? keep_first : 0;   // without a window every key is seen anyway
   LYP_REQUIRE(n_parts >= 1 && n_parts <= kPrefillPartsMost && (n_parts == 1 || (part_o && part_ml)),
               "attn_prefill: %d parts of the keys (at most %d, with a workspace)", n_parts, kPrefillPartsMost);
   if (n_tiles == 0) return 0;
@@ -1340,7 +1380,8 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
     dim3 grid(n_tiles*(64 / kQW), nkv * head_groups);                                                      \
     attn_prefill_kernel<T, GH, QB><<<grid, 256, 0, stream>>>(                                               \
         static_cast<const T*>(q), q_stride, static_cast<T*>(out), out_stride, kpool, vpool, block_tables,   \
-        max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window, scale_log2);         \
+        max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window, scale_log2, keep,    \
+        sink);                                                                                              \
   } while (0)
 #define LYP_PREFILL_T(T)                    \
   do {                                      \
@@ -1350,7 +1391,8 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   } while (0)
   constexpr int kQB4 = LYP_PREFILL_QB;
 #if LYP_HEAD_DIM % 32 == 0 && !defined(LYP_PREFILL_NARROW)
-  if (dtype == kBF16 && q_stride % 8 == 0 && bs % 16 == 0) {
+  // (the walk of the wide kernel knows no kept first tokens: a window with some takes the kernel above)
+  if (dtype == kBF16 && q_stride % 8 == 0 && bs % 16 == 0 && keep == 0) {
     // Bit 0 of `pair` is the caller's word on whether the tiles differ much in the keys they see
     // (0: no); bit 1 forbids the two sets of waves per unit (for tests and measurements).
     // Units (workgroups before pairing) beyond one per compute unit share compute units anyway;
@@ -1359,7 +1401,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   attn_prefill_wide_kernel<GH, NW, KS><<<grid, NW * KS * kWave, 0, stream>>>(                                 \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), out_stride, kpool, vpool,           \
       block_tables, max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window,            \
-      scale_log2, paired, part_o, part_ml, n_parts)
+      scale_log2, sink, paired, part_o, part_ml, n_parts)
     // Two sets of waves per unit while the launch has at most `kSplitBelow` workgroups per
     // compute unit: its time is then that of the unit with most keys, not of the sum.
 #define LYP_PREFILL_WIDE(GH, NW)                                                                              \
@@ -1384,7 +1426,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
 #undef LYP_PREFILL_WIDE_KS
     if (n_parts > 1)
       attn_merge_parts_kernel<bf16_t><<<dim3(nh, 64, n_tiles), 64, 0, stream>>>(
-          part_o, part_ml, n_parts, q_start, tile_seq, tile_q0, static_cast<bf16_t*>(out), out_stride, nh);
+          part_o, part_ml, n_parts, q_start, tile_seq, tile_q0, static_cast<bf16_t*>(out), out_stride, nh, sink);
     LYP_LAUNCH_CHECK("attn_prefill");
     return 0;
   }
@@ -1408,9 +1450,11 @@ int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, cons
                     const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
                     const int32_t* q_start, const int32_t* ctx_len, const int32_t* dec_seqs, int n_seqs,
                     float* part_o, float* part_ml, int max_parts, int part_keys, int nh, int nkv, int bs,
-                    int window, float scale, hipStream_t stream) {
+                    int window, float scale, int keep_first, const float* sink, hipStream_t stream) {
   if (check_common("attn_decode", nh, nkv, bs, max_blocks, q_stride, out_stride, window)) return -1;
-  LYP_REQUIRE(n_seqs >= 0 && max_parts > 0, "attn_decode: %d requests, %d partitions", n_seqs, max_parts);
+  LYP_REQUIRE(n_seqs >= 0 && max_parts > 0 && keep_first >= 0, "attn_decode: %d requests, %d partitions, %d kept",
+              n_seqs, max_parts, keep_first);
+  const int keep = window > 0 ? keep_first : 0;
   if (n_seqs == 0) return 0;
   const int g = nh / nkv;
   const int col_groups = (g + 15) / 16;
@@ -1429,7 +1473,7 @@ int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, cons
   attn_decode_kernel<T, WHOLE><<<grid, kDecodeWaves * kWave, lds, stream>>>(                            \
       static_cast<const T*>(q), q_stride, kpool, vpool, block_tables, max_blocks, q_start, ctx_len,      \
       dec_seqs, part_o, part_ml, max_parts, keys_per_wave, nh, nkv, bs, window, scale_log2,              \
-      static_cast<T*>(out), out_stride)
+      static_cast<T*>(out), out_stride, keep, sink)
 #define LYP_DECODE_T(T)                                                                                  \
   do {                                                                                                   \
     if (whole) {                                                                                         \
@@ -1438,7 +1482,7 @@ int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, cons
       LYP_DECODE(T, false);                                                                              \
       attn_combine_kernel<T><<<cgrid, 64, 0, stream>>>(part_o, part_ml, max_parts, q_start, ctx_len,     \
                                                        dec_seqs, static_cast<T*>(out), out_stride, nh,   \
-                                                       window, part_keys);                               \
+                                                       window, part_keys, keep, sink);                   \
     }                                                                                                    \
   } while (0)
   if (dtype == kF32) {

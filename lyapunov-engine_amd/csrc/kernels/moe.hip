@@ -1,0 +1,441 @@
+// A feed-forward that sends every token to a few of many small experts.
+//
+//   route      per token: router logits (float, computed by a 32-bit product) plus
+//              a bias, the `top` largest, and the softmax over those alone.
+//   sort       the (token, choice) pairs in order of their expert: where each
+//              expert's run starts, which pair stands at each place, the place
+//              of each pair, and the list of row tiles (expert, first place) the
+//              products walk.  One workgroup; the order inside a run is that of
+//              the pairs, whatever the timing.  Nothing goes back to the host: the
+//              products' grids are sized for the most tiles there can be.
+//   product    a tile of one expert's rows times a tile of that expert's matrix,
+//              on the matrix cores, through LDS.  GATED: rows are gathered from
+//              the step's activations by token, the gate's and the up
+//              projection's columns are computed side by side and the epilogue
+//              writes  min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1).
+//              Otherwise rows are read by place and the product is stored.
+//   combine    out[t] = addend[t] + shared[t] + sum_k weight[t, k] * y[place(t, k)],
+//              in 32-bit, in the order of k.
+//
+// Every row's sums run over the inner dimension in the same order wherever the
+// row stands in its tile, so a token's result does not depend on what else is in
+// the batch.
+#include <algorithm>
+
+#include "common.h"
+
+namespace lyp {
+
+constexpr int kRouteRegs = 8;            // experts per lane: up to 64 * 8 experts
+constexpr int kMostExperts = 64 * kRouteRegs;
+constexpr int kMostTop = 32;
+
+// z [rows, E] float logits without bias.  One wave per row.
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ bias,
+                                                        int rows, int E, int top, int32_t* __restrict__ idx,
+                                                        float* __restrict__ wgt) {
+  const int lane = threadIdx.x % kWave;
+  const int row = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (row >= rows) return;
+  float v[kRouteRegs];
+#pragma unroll
+  for (int r = 0; r < kRouteRegs; ++r) {
+    const int e = lane + kWave * r;
+    v[r] = e < E ? z[static_cast<size_t>(row) * E + e] + (bias != nullptr ? bias[e] : 0.f) : LYP_NEG_INF;
+  }
+  float chosen_v = 0.f;      // lane k keeps the k-th choice
+  int chosen_e = 0;
+  for (int k = 0; k < top; ++k) {
+    ArgMax best{LYP_NEG_INF, 0x7fffffff};
+#pragma unroll
+    for (int r = 0; r < kRouteRegs; ++r) best = better(best, ArgMax{v[r], lane + kWave * r});
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+      ArgMax o{__shfl_xor(best.v, off, kWave), __shfl_xor(best.i, off, kWave)};
+      best = better(best, o);
+    }
+#pragma unroll
+    for (int r = 0; r < kRouteRegs; ++r)
+      if (lane + kWave * r == best.i) v[r] = LYP_NEG_INF;
+    if (lane == k) {
+      chosen_v = best.v;
+      chosen_e = best.i;
+    }
+  }
+  const float m = __shfl(chosen_v, 0, kWave);      // the first choice is the largest
+  const float p = lane < top ? expf(chosen_v - m) : 0.f;
+  const float total = wave_sum(p);
+  if (lane < top) {
+    idx[static_cast<size_t>(row) * top + lane] = chosen_e;
+    wgt[static_cast<size_t>(row) * top + lane] = p / total;
+  }
+}
+
+constexpr int kSortThreads = 1024;
+constexpr int kSortWaves = kSortThreads / kWave;
+
+__global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
+    const int32_t* __restrict__ idx, int P, int E, int tile_rows, int32_t* __restrict__ expert_off,
+    int32_t* __restrict__ sorted_pair, int32_t* __restrict__ place_of, int32_t* __restrict__ tile_expert,
+    int32_t* __restrict__ tile_row0, int32_t* __restrict__ n_tiles) {
+  extern __shared__ int32_t s_sort[];
+  int32_t* cnt = s_sort;               // [E]
+  int32_t* base = cnt + E;             // [E]
+  int32_t* tbase = base + E;           // [E + 1]
+  int32_t* wcnt = tbase + E + 1;       // [kSortWaves][E]
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  for (int e = tid; e < E; e += kSortThreads) cnt[e] = 0;
+  __syncthreads();
+  for (int p = tid; p < P; p += kSortThreads) atomicAdd(&cnt[idx[p]], 1);   // integer counts: no order to depend on
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0, tiles = 0;
+    for (int e = 0; e < E; ++e) {
+      base[e] = run;
+      tbase[e] = tiles;
+      run += cnt[e];
+      tiles += (cnt[e] + tile_rows - 1) / tile_rows;
+    }
+    tbase[E] = tiles;
+    n_tiles[0] = tiles;
+  }
+  __syncthreads();
+  for (int e = tid; e <= E; e += kSortThreads) expert_off[e] = e < E ? base[e] : P;
+  for (int e = tid; e < E; e += kSortThreads) {
+    const int n = tbase[e + 1] - tbase[e];
+    for (int i = 0; i < n; ++i) {
+      tile_expert[tbase[e] + i] = e;
+      tile_row0[tbase[e] + i] = base[e] + i * tile_rows;
+    }
+  }
+  for (int p0 = 0; p0 < P; p0 += kSortThreads) {
+    __syncthreads();
+    for (int i = tid; i < kSortWaves * E; i += kSortThreads) wcnt[i] = 0;
+    __syncthreads();
+    const int p = p0 + tid;
+    const int e = p < P ? idx[p] : -1;
+    int rank = 0;
+    bool last = true;
+    for (int l = 0; l < kWave; ++l) {
+      const int el = __shfl(e, l, kWave);
+      if (el == e) {
+        if (l < lane) ++rank;
+        if (l > lane) last = false;
+      }
+    }
+    if (e >= 0 && last) wcnt[wave * E + e] = rank + 1;
+    __syncthreads();
+    if (e >= 0) {
+      int at = base[e] + rank;
+      for (int w = 0; w < wave; ++w) at += wcnt[w * E + e];
+      sorted_pair[at] = p;
+      place_of[p] = at;
+    }
+    __syncthreads();
+    for (int x = tid; x < E; x += kSortThreads) {
+      int add = 0;
+      for (int w = 0; w < kSortWaves; ++w) add += wcnt[w * E + x];
+      base[x] += add;
+    }
+  }
+}
+
+// ------------------------------------------------------------------- product
+// grid (most tiles, column tiles); 256 threads.  MB 16-row blocks of rows and
+// 64 output columns per workgroup; a wave takes one row block and 4 / (4 / MB)
+// column blocks (MB = 4), or the one row block and one column block (MB = 1).
+template <typename T, int MB, bool GATED, typename TO>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(
+    const T* __restrict__ a, int lda, const T* __restrict__ w, long long w_expert_stride, int ldw,
+    TO* __restrict__ out, int ldo, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
+    const int32_t* __restrict__ n_tiles, const int32_t* __restrict__ expert_off,
+    const int32_t* __restrict__ sorted_pair, int top, int N, int K, int up_offset, float limit, float alpha,
+    int vec_ok) {
+  using MW = Mma16Wide<T>;
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int KT = 32;
+  constexpr int LD = KT + (sizeof(T) == 2 ? 8 : 4);   // padded row: 16-byte reads of 16 rows fall into distinct banks
+  constexpr int TM = 16 * MB, TN = 64;
+  constexpr int BROWS = GATED ? 2 * TN : TN;
+  constexpr int WM = MB, WN = 4 / MB, CB = 4 / WN;
+  constexpr int STEPS = KT / (4 * MW::kElems);
+  constexpr int A_PER = (TM * KT / VEC + 255) / 256, B_PER = (BROWS * KT / VEC + 255) / 256;
+  typedef T VecT __attribute__((ext_vector_type(VEC)));
+  __shared__ __attribute__((aligned(16))) T As[TM * LD];
+  __shared__ __attribute__((aligned(16))) T Bs[BROWS * LD];
+
+  const int tile = blockIdx.x;
+  if (tile >= n_tiles[0]) return;
+  const int e = tile_expert[tile];
+  const int row0 = tile_row0[tile];
+  const int row_end = expert_off[e + 1];
+  const int c0 = blockIdx.y * TN;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave % WM, wn = wave / WM;
+  const T* we = w + static_cast<size_t>(e) * w_expert_stride;
+
+  // where this thread's pieces of the two tiles come from
+  const T* a_src[A_PER];
+  int a_k[A_PER], a_lds[A_PER];
+#pragma unroll
+  for (int n = 0; n < A_PER; ++n) {
+    const int v = tid + n * 256;
+    const int r = v / (KT / VEC), kc = (v % (KT / VEC)) * VEC;
+    a_k[n] = kc;
+    a_lds[n] = r * LD + kc;
+    a_src[n] = nullptr;
+    if (v < TM * KT / VEC && row0 + r < row_end) {
+      const int place = row0 + r;
+      const int src_row = GATED ? sorted_pair[place] / top : place;
+      a_src[n] = a + static_cast<size_t>(src_row) * lda;
+    }
+    if (v >= TM * KT / VEC) a_lds[n] = -1;
+  }
+  const T* b_src[B_PER];
+  int b_k[B_PER], b_lds[B_PER];
+#pragma unroll
+  for (int n = 0; n < B_PER; ++n) {
+    const int v = tid + n * 256;
+    const int r = v / (KT / VEC), kc = (v % (KT / VEC)) * VEC;
+    b_k[n] = kc;
+    b_lds[n] = v < BROWS * KT / VEC ? r * LD + kc : -1;
+    b_src[n] = nullptr;
+    if (v < BROWS * KT / VEC) {
+      const int col = c0 + r % TN;
+      if (col < N) b_src[n] = we + static_cast<size_t>(col + (GATED && r >= TN ? up_offset : 0)) * ldw;
+    }
+  }
+  auto fetch = [&](const T* src, int k) {
+    VecT x;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) x[i] = from_f32<T>(0.f);
+    if (src != nullptr) {
+      if (vec_ok && k + VEC <= K) {
+        x = *reinterpret_cast<const VecT*>(src + k);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+          if (k + i < K) x[i] = src[k + i];
+      }
+    }
+    return x;
+  };
+  VecT a_reg[A_PER], b_reg[B_PER];
+  auto load = [&](int k0) {
+#pragma unroll
+    for (int n = 0; n < A_PER; ++n) a_reg[n] = fetch(a_src[n], k0 + a_k[n]);
+#pragma unroll
+    for (int n = 0; n < B_PER; ++n) b_reg[n] = fetch(b_src[n], k0 + b_k[n]);
+  };
+  auto stash = [&] {
+#pragma unroll
+    for (int n = 0; n < A_PER; ++n)
+      if (a_lds[n] >= 0) *reinterpret_cast<VecT*>(As + a_lds[n]) = a_reg[n];
+#pragma unroll
+    for (int n = 0; n < B_PER; ++n)
+      if (b_lds[n] >= 0) *reinterpret_cast<VecT*>(Bs + b_lds[n]) = b_reg[n];
+  };
+
+  f32x4 acc[CB], acc_up[GATED ? CB : 1];
+#pragma unroll
+  for (int c = 0; c < CB; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < (GATED ? CB : 1); ++c) acc_up[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  load(0);
+  stash();
+  __syncthreads();
+  for (int k0 = 0; k0 < K; k0 += KT) {
+    const bool more = k0 + KT < K;
+    if (more) load(k0 + KT);
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int kk = s * 4 * MW::kElems + (lane / 16) * MW::kElems;
+      const typename MW::Frag xf = *reinterpret_cast<const typename MW::Frag*>(As + (wm * 16 + lane % 16) * LD + kk);
+#pragma unroll
+      for (int c = 0; c < CB; ++c) {
+        const int brow = (wn * CB + c) * 16 + lane % 16;
+        const typename MW::Frag wf = *reinterpret_cast<const typename MW::Frag*>(Bs + brow * LD + kk);
+        acc[c] = MW::mma(wf, xf, acc[c]);
+        if constexpr (GATED) {
+          const typename MW::Frag uf = *reinterpret_cast<const typename MW::Frag*>(Bs + (TN + brow) * LD + kk);
+          acc_up[c] = MW::mma(uf, xf, acc_up[c]);
+        }
+      }
+    }
+    __syncthreads();
+    if (more) {
+      stash();
+      __syncthreads();
+    }
+  }
+
+  // lane l: token row wm * 16 + l % 16, features (wn * CB + c) * 16 + 4 * (l / 16) + {0..3}
+  const int place = row0 + wm * 16 + lane % 16;
+  if (place >= row_end) return;
+  TO* orow = out + static_cast<size_t>(place) * ldo;
+#pragma unroll
+  for (int c = 0; c < CB; ++c) {
+    const int col = c0 + (wn * CB + c) * 16 + 4 * (lane / 16);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (col + i >= N) continue;
+      float y = acc[c][i];
+      if constexpr (GATED) {
+        const float g = fminf(y, limit);
+        const float u = fminf(fmaxf(acc_up[c][i], -limit), limit);
+        y = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+      }
+      orow[col + i] = from_f32<TO>(y);
+    }
+  }
+}
+
+// gate_up [rows, 2 I] (gates first) -> out [rows, I], the experts' activation
+template <typename T>
+__global__ void glu_clamped_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int rows, int I, float limit,
+                                   float alpha) {
+  const size_t total = static_cast<size_t>(rows) * I;
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const size_t r = i / I, c = i % I;
+    const float g = fminf(to_f32(gate_up[r * 2 * I + c]), limit);
+    const float u = fminf(fmaxf(to_f32(gate_up[r * 2 * I + I + c]), -limit), limit);
+    out[i] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+  }
+}
+
+// out [rows, H] float = addend + shared + sum_k wgt[row, k] * y[place_of[row * top + k]]
+template <typename T>
+__global__ void moe_combine_kernel(const T* __restrict__ y, const int32_t* __restrict__ place_of,
+                                   const float* __restrict__ wgt, int top, const T* __restrict__ addend,
+                                   const T* __restrict__ shared, float* __restrict__ out, int rows, int H) {
+  const int row = blockIdx.x;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    float v = 0.f;
+    if (addend != nullptr) v += to_f32(addend[static_cast<size_t>(row) * H + c]);
+    if (shared != nullptr) v += to_f32(shared[static_cast<size_t>(row) * H + c]);
+    for (int k = 0; k < top; ++k) {
+      const int at = place_of[static_cast<size_t>(row) * top + k];
+      v += wgt[static_cast<size_t>(row) * top + k] * to_f32(y[static_cast<size_t>(at) * H + c]);
+    }
+    out[static_cast<size_t>(row) * H + c] = v;
+  }
+}
+
+}  // namespace lyp
+
+using namespace lyp;
+
+extern "C" {
+
+int lyp_moe_most_experts() { return kMostExperts; }
+
+int lyp_moe_route(const float* z, const float* bias, int rows, int E, int top, int32_t* idx, float* wgt,
+                  hipStream_t stream) {
+  LYP_REQUIRE(rows >= 0 && E > 0 && E <= kMostExperts && top > 0 && top <= E && top <= kMostTop,
+              "moe_route: %d rows, %d experts (at most %d), %d chosen (at most %d)", rows, E, kMostExperts, top,
+              kMostTop);
+  if (rows == 0) return 0;
+  moe_route_kernel<<<(rows + 3) / 4, 256, 0, stream>>>(z, bias, rows, E, top, idx, wgt);
+  LYP_LAUNCH_CHECK("moe_route");
+  return 0;
+}
+
+// Rows per tile the products had better use for `pairs` pairs over E experts, and the most tiles
+// there can then be (the products' grid).
+int lyp_moe_tile_rows(int pairs, int E) { return pairs >= 32 * E ? 64 : 16; }
+int lyp_moe_most_tiles(int pairs, int E, int tile_rows) {
+  return (pairs + tile_rows - 1) / tile_rows + std::min(E, pairs);
+}
+
+int lyp_moe_sort(const int32_t* idx, int pairs, int E, int tile_rows, int32_t* expert_off, int32_t* sorted_pair,
+                 int32_t* place_of, int32_t* tile_expert, int32_t* tile_row0, int32_t* n_tiles, hipStream_t stream) {
+  LYP_REQUIRE(pairs >= 0 && E > 0 && E <= kMostExperts && (tile_rows == 16 || tile_rows == 64),
+              "moe_sort: %d pairs, %d experts, tiles of %d rows", pairs, E, tile_rows);
+  const size_t lds = sizeof(int32_t) * (3 * E + 1 + kSortWaves * E);
+  moe_sort_kernel<<<1, kSortThreads, lds, stream>>>(idx, pairs, E, tile_rows, expert_off, sorted_pair, place_of,
+                                                    tile_expert, tile_row0, n_tiles);
+  LYP_LAUNCH_CHECK("moe_sort");
+  return 0;
+}
+
+// gated != 0: a [tokens, K] gathered by token, w [E][2 N rows: gates, then ups][K], out [pairs, N] in the
+// operands' type.  gated == 0: a [pairs, K] by place, w [E][N][K], out [pairs, N] in the operands' type.
+int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_stride, int ldw, void* out, int ldo,
+                 int dtype, int gated, const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* n_tiles,
+                 int most_tiles, int tile_rows, const int32_t* expert_off, const int32_t* sorted_pair, int top, int N,
+                 int K, float limit, float alpha, hipStream_t stream) {
+  LYP_REQUIRE(N > 0 && K > 0 && lda >= K && ldw >= K && ldo >= N && top > 0 && most_tiles >= 0,
+              "moe_gemm: bad sizes N=%d K=%d lda=%d ldw=%d ldo=%d", N, K, lda, ldw, ldo);
+  LYP_REQUIRE(tile_rows == 16 || tile_rows == 64, "moe_gemm: tiles of %d rows", tile_rows);
+  if (most_tiles == 0) return 0;
+  const int col_tiles = (N + 63) / 64;
+  LYP_REQUIRE(col_tiles <= 65535, "moe_gemm: too many columns for one launch");
+  const int esz = dtype == kF32 ? 4 : 2;
+  const int vec = 16 / esz;
+  const int vec_ok = lda % vec == 0 && ldw % vec == 0 && w_expert_stride % vec == 0 &&
+                     reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
+  dim3 grid(most_tiles, col_tiles);
+#define LYP_MOE(T, MB, G)                                                                                       \
+  moe_gemm_kernel<T, MB, G, T><<<grid, 256, 0, stream>>>(                                                       \
+      static_cast<const T*>(a), lda, static_cast<const T*>(w), w_expert_stride, ldw, static_cast<T*>(out), ldo, \
+      tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok)
+#define LYP_MOE_T(T)                                 \
+  do {                                               \
+    if (tile_rows == 64) {                           \
+      if (gated) LYP_MOE(T, 4, true);                \
+      else LYP_MOE(T, 4, false);                     \
+    } else {                                         \
+      if (gated) LYP_MOE(T, 1, true);                \
+      else LYP_MOE(T, 1, false);                     \
+    }                                                \
+  } while (0)
+  if (dtype == kF32) LYP_MOE_T(float);
+  else if (dtype == kBF16) LYP_MOE_T(bf16_t);
+  else LYP_REQUIRE(false, "moe_gemm: unknown dtype %d", dtype);
+#undef LYP_MOE_T
+#undef LYP_MOE
+  LYP_LAUNCH_CHECK("moe_gemm");
+  return 0;
+}
+
+int lyp_glu_clamped(const void* gate_up, void* out, int dtype, int rows, int I, float limit, float alpha,
+                    hipStream_t stream) {
+  LYP_REQUIRE(rows >= 0 && I > 0, "glu_clamped: bad sizes");
+  if (rows == 0) return 0;
+  const long long total = static_cast<long long>(rows) * I;
+  const int blocks = static_cast<int>(std::min<long long>((total + 255) / 256, 8192));
+  if (dtype == kF32)
+    glu_clamped_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(gate_up),
+                                                          static_cast<float*>(out), rows, I, limit, alpha);
+  else if (dtype == kBF16)
+    glu_clamped_kernel<bf16_t><<<blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(gate_up),
+                                                           static_cast<bf16_t*>(out), rows, I, limit, alpha);
+  else
+    LYP_REQUIRE(false, "glu_clamped: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("glu_clamped");
+  return 0;
+}
+
+int lyp_moe_combine(const void* y, const int32_t* place_of, const float* wgt, int top, const void* addend,
+                    const void* shared, float* out, int dtype, int rows, int H, hipStream_t stream) {
+  LYP_REQUIRE(rows >= 0 && H > 0 && top > 0, "moe_combine: bad sizes");
+  if (rows == 0) return 0;
+  const int threads = H >= 1024 ? 256 : 128;
+  if (dtype == kF32)
+    moe_combine_kernel<float><<<rows, threads, 0, stream>>>(static_cast<const float*>(y), place_of, wgt, top,
+                                                            static_cast<const float*>(addend),
+                                                            static_cast<const float*>(shared), out, rows, H);
+  else if (dtype == kBF16)
+    moe_combine_kernel<bf16_t><<<rows, threads, 0, stream>>>(static_cast<const bf16_t*>(y), place_of, wgt, top,
+                                                             static_cast<const bf16_t*>(addend),
+                                                             static_cast<const bf16_t*>(shared), out, rows, H);
+  else
+    LYP_REQUIRE(false, "moe_combine: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("moe_combine");
+  return 0;
+}
+
+}  // extern "C"

@@ -42,10 +42,10 @@ const char* lyp_rt_last_error() { return g_error.c_str(); }
 
 // ------------------------------------------------------------- cache manager
 void* lyp_cache_create(int num_groups, const int* num_pages, const int* page_size, const int* window,
-                       int num_state_slots) {
+                       const int* keep_first, int num_state_slots) {
   try {
     std::vector<lyp::GroupSpec> groups(num_groups);
-    for (int g = 0; g < num_groups; ++g) groups[g] = {num_pages[g], page_size[g], window[g]};
+    for (int g = 0; g < num_groups; ++g) groups[g] = {num_pages[g], page_size[g], window[g], keep_first ? keep_first[g] : 0};
     return new CacheManager(std::move(groups), num_state_slots);
   } catch (const std::exception& e) {
     g_error = e.what();

@@ -15,8 +15,8 @@ CacheManager::CacheManager(std::vector<GroupSpec> groups, int num_state_slots)
     : groups_(std::move(groups)), num_state_slots_(num_state_slots) {
   if (groups_.empty()) throw std::invalid_argument("cache manager needs at least one group");
   for (const auto& g : groups_) {
-    if (g.num_pages <= 0 || g.page_size <= 0 || g.window < 0)
-      throw std::invalid_argument("cache group needs num_pages > 0, page_size > 0, window >= 0");
+    if (g.num_pages <= 0 || g.page_size <= 0 || g.window < 0 || g.keep_first < 0)
+      throw std::invalid_argument("cache group needs num_pages > 0, page_size > 0, window >= 0, keep_first >= 0");
   }
   if (num_state_slots_ <= 0) throw std::invalid_argument("cache manager needs at least one state slot");
   reset();
@@ -59,7 +59,8 @@ int CacheManager::pages_held_at_most(int g, int len, int portion) const {
   const GroupSpec& spec = groups_.at(g);
   const int all = ceil_div(len, spec.page_size);
   if (spec.window <= 0) return all;
-  return std::min(all, ceil_div(spec.window + std::max(portion, 1), spec.page_size) + 1);
+  return std::min(all, ceil_div(spec.window + std::max(portion, 1), spec.page_size) + 1 +
+                           ceil_div(spec.keep_first, spec.page_size));
 }
 
 int CacheManager::max_length(int64_t id) const {
@@ -120,7 +121,8 @@ void CacheManager::commit(int64_t id, int new_len) {
     // The next token sits at position new_len and sees keys > new_len - window.
     const int first_needed = new_len - spec.window + 1;
     auto& table = r.tables[g];
-    for (size_t i = 0; i < table.size(); ++i) {
+    // pages that hold one of the kept first keys stay
+    for (size_t i = ceil_div(spec.keep_first, spec.page_size); i < table.size(); ++i) {
       if (static_cast<int>(i + 1) * spec.page_size > first_needed) break;
       if (table[i] >= 0) {
         release_page(g, table[i]);

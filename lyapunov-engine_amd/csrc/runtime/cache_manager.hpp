@@ -27,6 +27,7 @@ struct GroupSpec {
   int num_pages = 0;
   int page_size = 16;
   int window = 0;  // 0: every key is kept; W > 0: a token sees keys (pos - W, pos]
+  int keep_first = 0;  // with a window: a request's first keep_first keys stay visible, so their pages are never given back
 };
 
 class CacheManager {

@@ -35,7 +35,7 @@ static int one_round(std::mt19937& rng) {
   const int pages = pick(6, 40);
   const int window = pick(0, 2) == 0 ? pick(2, 3 * page) : 0;
   std::vector<GroupSpec> groups{{pages, page, 0}};
-  if (window) groups.push_back({pages, page, window});
+  if (window) groups.push_back({pages, page, window, pick(0, 1) ? pick(1, 2 * page) : 0});   // some windows keep first tokens
   CacheManager cache(groups, pick(2, 6));
   SchedulerConfig cfg;
   cfg.max_num_seqs = pick(1, 6);

@@ -30,7 +30,8 @@ class EngineCore:
         self.block_size = block_size
         layout = model.cache_layout()
         sizes = self.group_sizes(layout, num_blocks, block_size, cache_groups)
-        groups = [GroupConfig(pages, size, gl.spec.window) for (pages, size), gl in zip(sizes, layout.groups)]
+        groups = [GroupConfig(pages, size, gl.spec.window, gl.spec.keep_first)
+                  for (pages, size), gl in zip(sizes, layout.groups)]
         # A model without keys and values (state only) still gets a group, so
         # that requests have a length and the manager one code path.
         self.cache = CacheManager(groups or [GroupConfig(num_blocks, block_size, 0)], num_state_slots)

@@ -23,7 +23,8 @@ class TraceReplayer:
         num_blocks = max(1, -(-max_tokens // block_size))
         self.core = EngineCore.from_folder(model_dir, dtype=dtype, device=device, num_blocks=num_blocks,
                                            block_size=block_size, num_state_slots=MAX_LIVE_REQUESTS,
-                                           cache_groups=cache_groups)
+                                           cache_groups=cache_groups,
+                                           max_model_len=num_blocks * block_size)   # no request outgrows the pool
         self._ids: dict = {}
         self._next_id = 0
 

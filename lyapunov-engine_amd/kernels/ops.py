@@ -106,6 +106,24 @@ def core() -> ctypes.CDLL:
         lib.lyp_latent_attn_rows.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                              c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                              c_void_p]
+        lib.lyp_qk_norm_rope_kv.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int,
+                                            c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                            c_void_p]
+        lib.lyp_attn_rows.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p,
+                                      c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p, c_int, c_int, c_int,
+                                      c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_stream_add.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_longlong, c_void_p]
+        lib.lyp_moe_route.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+        lib.lyp_moe_tile_rows.argtypes = [c_int, c_int]
+        lib.lyp_moe_most_tiles.argtypes = [c_int, c_int, c_int]
+        lib.lyp_moe_sort.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     c_void_p, c_void_p]
+        lib.lyp_moe_gemm.argtypes = [c_void_p, c_int, c_void_p, c_longlong, c_int, c_void_p, c_int, c_int, c_int,
+                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                                     c_float, c_float, c_void_p]
+        lib.lyp_glu_clamped.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p]
+        lib.lyp_moe_combine.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                        c_int, c_void_p]
         _core = lib
     return _core
 
@@ -119,11 +137,11 @@ def attention_lib(head_dim: int) -> ctypes.CDLL:
             raise KernelError(f"attention library for head size {head_dim} reports {lib.lyp_attn_head_dim()}")
         lib.lyp_attn_prefill.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                         c_float, c_int, c_void_p, c_void_p, c_int, c_void_p]
+                                         c_float, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]
         lib.lyp_attn_prefill_plan.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int]
         lib.lyp_attn_decode.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                         c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-                                        c_int, c_int, c_int, c_float, c_void_p]
+                                        c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p]
         lib.lyp_attn_decode_plan.argtypes = [c_int, c_int, c_int, c_int]
         _attn[head_dim] = lib
     return lib
@@ -1148,6 +1166,13 @@ def attn_prefill_plan(n_tiles: int, max_keys: int, num_heads: int, num_kv_heads:
                                                          page_size)
 
 
+def _sink_check(sink, num_heads: int) -> None:
+    if sink is not None:
+        _dev(sink)
+        if sink.dtype != torch.float32 or sink.numel() != num_heads:
+            raise KernelError(f"attention: the sinks are float, one per query head, not {tuple(sink.shape)} {sink.dtype}")
+
+
 def _attn_check(q, out, kpool, vpool, block_tables, nh, nkv, hd):
     _dev(out, kpool, vpool, block_tables)
     n_pages, bs = kpool.shape[0], kpool.shape[2]
@@ -1167,7 +1192,8 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
                  tile_q0: torch.Tensor, n_tiles: int, *, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: int = 0, scale: float | None = None, pair: bool | None = None,
                  split: bool = True, parts: int = 1, part_o: torch.Tensor | None = None,
-                 part_ml: torch.Tensor | None = None) -> torch.Tensor:
+                 part_ml: torch.Tensor | None = None, keep_first: int = 0,
+                 sink: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache (which already
     holds their own keys).  q is a view [T, >= nh * hd] whose first nh * hd
     columns are the query heads; a tile is 64 new tokens of one request, and
@@ -1179,7 +1205,11 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
     > 1 (see ``attn_prefill_plan``) cuts every tile's keys into that many runs
     for workgroups of their own; it needs float workspaces ``part_o`` of
     n_tiles * 64 * heads * parts * head_dim and ``part_ml`` of n_tiles * 64 *
-    heads * parts * 2 elements."""
+    heads * parts * 2 elements.  With a window, ``keep_first`` first tokens of a
+    request stay visible whatever the distance; ``sink`` (float, one per query
+    head) is a score without key or value that stands in the softmax's
+    denominator once."""
+    _sink_check(sink, num_heads)
     if not q.is_cuda or q.dim() != 2:
         raise KernelError("attention: q must be a 2-d GPU tensor")
     bs = _attn_check(q, out, kpool, vpool, block_tables, num_heads, num_kv_heads, head_dim)
@@ -1195,7 +1225,7 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
                                 _p(block_tables), block_tables.shape[1], _p(q_start), _p(ctx_len), _p(tile_seq),
                                 _p(tile_q0), n_tiles, num_heads, num_kv_heads, bs, window, scale,
                                 (1 if pair is None else int(bool(pair))) | (0 if split else 2), _p(part_o),
-                                _p(part_ml), parts, _stream()), lib)
+                                _p(part_ml), parts, int(keep_first), _p(sink), _stream()), lib)
     return out
 
 
@@ -1203,13 +1233,15 @@ def attn_decode(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: 
                 block_tables: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                 dec_seqs: torch.Tensor | None, n_seqs: int, part_o: torch.Tensor, part_ml: torch.Tensor,
                 max_parts: int, part_keys: int, *, num_heads: int, num_kv_heads: int, head_dim: int, window: int = 0,
-                scale: float | None = None) -> torch.Tensor:
+                scale: float | None = None, keep_first: int = 0, sink: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of requests that bring one new token each, split over
     partitions of the context and merged.  ``part_keys`` comes from
     ``attn_decode_plan``; the caller guarantees that no request's context
     exceeds ``max_parts * part_keys`` (the contexts live on the device and are
     not read here: keys beyond that many partitions would silently be left
-    out).  ``PagedAttention.decode_launch`` derives both from the step's bound."""
+    out).  ``PagedAttention.decode_launch`` derives both from the step's bound.
+    ``keep_first`` and ``sink``: as for ``attn_prefill``."""
+    _sink_check(sink, num_heads)
     if not q.is_cuda or q.dim() != 2:
         raise KernelError("attention: q must be a 2-d GPU tensor")
     bs = _attn_check(q, out, kpool, vpool, block_tables, num_heads, num_kv_heads, head_dim)
@@ -1223,7 +1255,172 @@ def attn_decode(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: 
     _check(lib.lyp_attn_decode(_p(q), q.stride(0), _p(out), out.stride(0), _p(kpool), _p(vpool), _code(q.dtype),
                                _p(block_tables), block_tables.shape[1], _p(q_start), _p(ctx_len), _p(dec_seqs),
                                n_seqs, _p(part_o), _p(part_ml), max_parts, part_keys, num_heads, num_kv_heads, bs,
-                               window, scale, _stream()), lib)
+                               window, scale, int(keep_first), _p(sink), _stream()), lib)
+    return out
+
+
+# ------------------------------- normed projections, windows with kept tokens, sinks
+def qk_norm_rope_kv(qkv: torch.Tensor, q_norm: torch.Tensor | None, k_norm: torch.Tensor | None, eps: float,
+                    positions: torch.Tensor, table: torch.Tensor | None, slots: torch.Tensor | None,
+                    kpool: torch.Tensor | None, vpool: torch.Tensor | None, *, num_heads: int, num_kv_heads: int,
+                    dim: int, vdim: int, page_size: int) -> None:
+    """qkv [T, (H + G) dim + G vdim]: one RMS norm over each token's whole query projection and one
+    over its whole key projection (``q_norm`` [H dim], ``k_norm`` [G dim], float; None: no norm),
+    rotation of the pairs (2i, 2i+1) of the first ``table.shape[1]`` values of every query and key
+    head by the token's position (table rows: cosines, then sines), queries back in place, keys and
+    values into the tokens' page slots (keys [pages, G, page, dim], values [pages, G, vdim, page])."""
+    _dev(qkv, q_norm, k_norm, positions, table, slots, kpool, vpool)
+    _f32(q_norm, k_norm, table)
+    T = qkv.shape[0]
+    H, G = num_heads, num_kv_heads
+    rot = 0 if table is None else table.shape[1]
+    if qkv.shape[1] != (H + G) * dim + G * vdim or positions.numel() != T or positions.dtype != torch.int32 or \
+            (q_norm is not None and q_norm.numel() != H * dim) or (k_norm is not None and k_norm.numel() != G * dim):
+        raise KernelError(f"qk_norm_rope_kv: qkv {tuple(qkv.shape)} for {H}+{G} heads of {dim}/{vdim}")
+    if slots is not None:
+        n_pages = kpool.shape[0]
+        if (slots.numel() != T or slots.dtype != torch.int32 or tuple(kpool.shape) != (n_pages, G, page_size, dim)
+                or tuple(vpool.shape) != (n_pages, G, vdim, page_size) or kpool.dtype != qkv.dtype
+                or vpool.dtype != qkv.dtype):
+            raise KernelError(f"qk_norm_rope_kv: pools {tuple(kpool.shape)} / {tuple(vpool.shape)} {kpool.dtype} do "
+                              f"not fit {G} heads of {dim}/{vdim}, pages of {page_size}, dtype {qkv.dtype}")
+    lib = core()
+    _check(lib.lyp_qk_norm_rope_kv(_p(qkv), qkv.stride(0), _code(qkv.dtype), _p(q_norm), _p(k_norm), float(eps),
+                                   _p(positions), _p(table), rot, _p(slots), _p(kpool), _p(vpool), T, H, G, dim, vdim,
+                                   page_size, _stream()), lib)
+
+
+def attn_rows(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_tables: torch.Tensor,
+              q_start: torch.Tensor, positions: torch.Tensor, ctx_len: torch.Tensor, *, num_heads: int,
+              num_kv_heads: int, dim: int, vdim: int, scale: float, window: int = 0, keep_first: int = 0,
+              sink: torch.Tensor | None = None) -> torch.Tensor:
+    """Attention of every row of the step over its request's pages for any key and value size: q a
+    view [T, >= H dim], out [T, H vdim].  A row at position p sees key j <= p when window == 0,
+    p - j < window or j < keep_first."""
+    _sink_check(sink, num_heads)
+    _dev(out, kpool, vpool, block_tables, q_start, positions, ctx_len)
+    n_pages, bs = kpool.shape[0], kpool.shape[2]
+    T = q.shape[0]
+    if (not q.is_cuda or q.stride(1) != 1 or q.stride(0) < num_heads * dim
+            or tuple(kpool.shape) != (n_pages, num_kv_heads, bs, dim) or tuple(vpool.shape) != (n_pages, num_kv_heads, vdim, bs)
+            or tuple(out.shape) != (T, num_heads * vdim) or len({q.dtype, out.dtype, kpool.dtype, vpool.dtype}) != 1
+            or block_tables.dtype != torch.int32 or block_tables.dim() != 2):
+        raise KernelError(f"attn_rows: q {tuple(q.shape)}, out {tuple(out.shape)}, pools {tuple(kpool.shape)} / "
+                          f"{tuple(vpool.shape)} for {num_heads}/{num_kv_heads} heads of {dim}/{vdim}")
+    lib = core()
+    _check(lib.lyp_attn_rows(_p(q), q.stride(0), _p(kpool), _p(vpool), _p(block_tables), block_tables.shape[1], bs,
+                             _p(q_start), _p(positions), _p(ctx_len), q_start.numel() - 1, _p(sink), float(scale),
+                             int(window), int(keep_first), _p(out), out.stride(0), _code(q.dtype), T, num_heads,
+                             num_kv_heads, dim, vdim, _stream()), lib)
+    return out
+
+
+def stream_add(h: torch.Tensor, a, b: torch.Tensor | None = None) -> None:
+    """h += a + b on the float residual stream: ``a`` what a layer left to be added (None, a tensor
+    [T, H], float partial sums [S, T, H] or a product still to be run), ``b`` a float tensor [T, H]."""
+    if isinstance(a, PendingLinear):
+        a = a.run()
+    _dev(h, a, b)
+    parts = 0
+    if a is not None:
+        parts = a.shape[0] if a.dim() == 3 else 1
+        if tuple(a.shape[-2:]) != tuple(h.shape) or (a.dim() == 3 and a.dtype != torch.float32):
+            raise KernelError(f"stream_add: {tuple(a.shape)} {a.dtype} onto {tuple(h.shape)}")
+    if h.dtype != torch.float32 or (b is not None and (b.dtype != torch.float32 or b.shape != h.shape)):
+        raise KernelError("stream_add: the stream and what is added to it whole are float and of one shape")
+    lib = core()
+    _check(lib.lyp_stream_add(_p(h), _p(a), _code(a.dtype) if a is not None else 0, parts, _p(b), h.numel(),
+                              _stream()), lib)
+
+
+# ------------------------------------------------------------ routed feed-forward
+def glu_clamped(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """[T, 2 I] (gates first) -> [T, I]: g = min(gate, limit), u = clamp(up, -limit, limit);
+    g * sigmoid(alpha * g) * (u + 1)."""
+    _dev(gate_up)
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
+    lib = core()
+    _check(lib.lyp_glu_clamped(_p(gate_up), _p(out), _code(gate_up.dtype), T, I, float(limit), float(alpha), _stream()), lib)
+    return out
+
+
+def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, top: int):
+    """float router logits [T, E] (+ bias) -> (experts int32 [T, top], weights float [T, top]): the
+    ``top`` largest (of equal ones the first) and the softmax over those alone."""
+    _dev(logits, bias)
+    _f32(logits, bias)
+    T, E = logits.shape
+    idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    wgt = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    lib = core()
+    _check(lib.lyp_moe_route(_p(logits), _p(bias), T, E, top, _p(idx), _p(wgt), _stream()), lib)
+    return idx, wgt
+
+
+class MoePlan:
+    """Where the (token, choice) pairs of a step stand once sorted by expert, on the device."""
+
+    def __init__(self, idx: torch.Tensor, E: int):
+        lib = core()
+        self.pairs, self.top, self.E = idx.numel(), idx.shape[1], E
+        self.tile_rows = lib.lyp_moe_tile_rows(self.pairs, E)
+        self.most_tiles = lib.lyp_moe_most_tiles(self.pairs, E, self.tile_rows)
+        # one allocation: expert offsets, pair at each place, place of each pair, tiles, their count
+        sizes = (E + 1, self.pairs, self.pairs, self.most_tiles, self.most_tiles, 1)
+        buf = torch.empty(sum(sizes), dtype=torch.int32, device=idx.device)
+        views, at = [], 0
+        for n in sizes:
+            views.append(buf[at:at + n])
+            at += n
+        self.expert_off, self.sorted_pair, self.place_of, self.tile_expert, self.tile_row0, self.n_tiles = views
+        _check(lib.lyp_moe_sort(_p(idx), self.pairs, E, self.tile_rows, _p(self.expert_off), _p(self.sorted_pair),
+                                _p(self.place_of), _p(self.tile_expert), _p(self.tile_row0), _p(self.n_tiles),
+                                _stream()), lib)
+
+
+def moe_sort(idx: torch.Tensor, num_experts: int) -> MoePlan:
+    _dev(idx)
+    if idx.dtype != torch.int32 or idx.dim() != 2:
+        raise KernelError("moe_sort: the chosen experts are int32 [tokens, top]")
+    return MoePlan(idx, num_experts)
+
+
+def moe_gemm(a: torch.Tensor, w: torch.Tensor, plan: MoePlan, *, gated: bool, limit: float = 0.0,
+             alpha: float = 0.0) -> torch.Tensor:
+    """One product per expert over the rows sorted to it.  gated: a [T, K] (rows gathered by token),
+    w [E, 2 N, K] (an expert's gate rows, then its up rows) -> [pairs, N], the gated activation of
+    ``glu_clamped`` applied.  Otherwise a [pairs, K] in sorted order, w [E, N, K] -> [pairs, N]."""
+    _dev(a, w)
+    E, rows, K = w.shape
+    N = rows // 2 if gated else rows
+    if a.dtype != w.dtype or a.shape[1] != K or E != plan.E or (not gated and a.shape[0] != plan.pairs):
+        raise KernelError(f"moe_gemm: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, {plan.pairs} pairs")
+    out = torch.empty((plan.pairs, N), dtype=a.dtype, device=a.device)
+    lib = core()
+    _check(lib.lyp_moe_gemm(_p(a), a.stride(0), _p(w), w.stride(0), w.stride(1), _p(out), out.stride(0), _code(a.dtype),
+                            int(gated), _p(plan.tile_expert), _p(plan.tile_row0), _p(plan.n_tiles), plan.most_tiles,
+                            plan.tile_rows, _p(plan.expert_off), _p(plan.sorted_pair), plan.top, N, K, float(limit),
+                            float(alpha), _stream()), lib)
+    return out
+
+
+def moe_combine(y: torch.Tensor, plan: MoePlan, weights: torch.Tensor, rows: int, addend: torch.Tensor | None = None,
+                shared: torch.Tensor | None = None) -> torch.Tensor:
+    """float [1, rows, H]: addend + shared + sum over a token's choices of weight * y[place of the
+    pair], added up in 32-bit in the order of the choices (one slice of partial sums, which a norm
+    adds to the residual stream)."""
+    _dev(y, weights, addend, shared)
+    H = y.shape[1]
+    for t in (addend, shared):
+        if t is not None and (tuple(t.shape) != (rows, H) or t.dtype != y.dtype):
+            raise KernelError(f"moe_combine: {tuple(t.shape)} {t.dtype} beside [{rows}, {H}] {y.dtype}")
+    if weights.dtype != torch.float32 or weights.numel() != plan.pairs or rows * plan.top != plan.pairs:
+        raise KernelError("moe_combine: weights do not fit the pairs")
+    out = torch.empty((1, rows, H), dtype=torch.float32, device=y.device)
+    lib = core()
+    _check(lib.lyp_moe_combine(_p(y), _p(plan.place_of), _p(weights), plan.top, _p(addend), _p(shared), _p(out),
+                               _code(y.dtype), rows, H, _stream()), lib)
     return out
 
 

@@ -179,8 +179,15 @@ class DecoderModel(Part):
         ``Logits`` (None if R == 0).
         ``caches[i]`` is the LayerCache of ``schedule[i]``."""
         h = self.embedding.forward(ctx, ctx.token_ids)
+        # calls that add the embedding's output again read it from a second copy (h itself moves on)
+        first = self.embedding.forward(ctx, ctx.token_ids) if any(c.reinject for c in self.schedule) else None
         delta = None
         for call, cache in zip(self.schedule, caches):
+            if call.reinject:
+                if isinstance(delta, ops.JoiningBranch):
+                    delta = delta.join(h)
+                ops.stream_add(h, delta, first)      # what was still to be added, and the embedding's rows
+                delta = None
             if call.shift is not None:
                 delta = ops.shifted(h, delta, self.stream_shift.row(call.shift))
             h, delta = self.layers[call.layer].forward(ctx, h, delta, cache)

@@ -111,13 +111,17 @@ class PagedSpec:
 
     tensors: tuple         # of PageTensor
     window: int = 0        # 0: every token is kept; W: a token needs the last W tokens' entries, its own included
+    keep_first: int = 0    # with a window: a token also needs the request's first keep_first entries
 
     @classmethod
-    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int = 0) -> "PagedSpec":
+    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int = 0, value_dim: Optional[int] = None,
+                        keep_first: int = 0) -> "PagedSpec":
         """The layout the attention kernels of this package read: keys
-        [heads][slot][head_dim], values [heads][head_dim][slot]."""
-        return cls((PageTensor("k", (num_kv_heads, SLOT, head_dim)), PageTensor("v", (num_kv_heads, head_dim, SLOT))),
-                   int(window))
+        [heads][slot][head_dim], values [heads][value_dim][slot] (``value_dim``
+        None: the keys' size)."""
+        vd = head_dim if value_dim is None else int(value_dim)
+        return cls((PageTensor("k", (num_kv_heads, SLOT, head_dim)), PageTensor("v", (num_kv_heads, vd, SLOT))),
+                   int(window), int(keep_first) if window else 0)
 
 
 @dataclass(frozen=True)

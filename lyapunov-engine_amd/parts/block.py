@@ -8,6 +8,8 @@ added.
 """
 from __future__ import annotations
 
+import torch
+
 from ..config.registry import BLOCKS, FEED_FORWARDS, FILTERS, MIXERS, NORMS
 from ..config.specs import LayerSpec
 from ..kernels import ops
@@ -92,6 +94,42 @@ class SandwichBlock(Block):
             return h, branch
         x = self.norm2.forward(ctx, h, branch)
         return h, self.norm2_out.branch(self.ffn.forward(ctx, x), self.mult)
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock(Block):
+    """One norm whose output both branches read: h += mixer(n) + ffn(n), n = norm1(h).  The
+    feed-forward branch may be absent (``LayerSpec.ffn`` None).  The sum of the two branches is
+    formed in 32-bit (by a feed-forward with ``takes_addend``, in its last kernel) and returned still
+    to be added; the norm that follows adds it to the stream."""
+
+    def __init__(self, spec: LayerSpec):
+        self.names = dict(spec.names)
+        self.norm1 = NORMS.build(spec.norm1)
+        self.mixer = MIXERS.build(spec.mixer)
+        self.ffn = FEED_FORWARDS.build(spec.ffn) if spec.ffn is not None else None
+        if spec.extra:
+            raise ValueError(f"the parallel arrangement has no parts {sorted(spec.extra)}")
+
+    def children(self):
+        n = self.names
+        out = {n["norm1"]: self.norm1, n["mixer"]: self.mixer}
+        if self.ffn is not None:
+            out[n["ffn"]] = self.ffn
+        return out
+
+    def forward(self, ctx: StepContext, h, delta, cache: LayerCache):
+        x = normed(self.norm1, None, ctx, h, delta)
+        a = self.mixer.forward(ctx, x, cache)
+        if self.ffn is None:
+            return h, a
+        if getattr(self.ffn, "takes_addend", False):
+            return h, self.ffn.forward(ctx, x, addend=a)
+        f = self.ffn.forward(ctx, x)
+        both = torch.zeros((ctx.T, h.shape[1]), dtype=torch.float32, device=h.device)
+        ops.stream_add(both, a)
+        ops.stream_add(both, f)
+        return h, both.view(1, ctx.T, h.shape[1])
 
 
 def normed(norm, consumer, ctx: StepContext, h, delta):

@@ -30,6 +30,8 @@ def rotary_inv_freq(dim: int, theta: float, scaling: Optional[dict] = None) -> t
     inv_freq = 1.0 / (theta ** (torch.arange(0, dim, 2).float() / dim))
     if not scaling or scaling.get("rope_type", "default") == "default":
         return inv_freq
+    if scaling["rope_type"] == "linear":      # every frequency divided by one constant
+        return inv_freq / float(scaling["factor"])
     if scaling["rope_type"] != "llama3":
         raise ValueError(f"rotary scaling {scaling['rope_type']!r} is not implemented")
     factor = float(scaling["factor"])
@@ -52,7 +54,10 @@ _TABLES: "weakref.WeakValueDictionary" = weakref.WeakValueDictionary()
 
 @POSITION_ENCODINGS.register("rope")
 class RotaryEncoding(PositionEncoding):
-    def __init__(self, dim: int, theta: float, max_position: int, scaling: Optional[dict] = None):
+    def __init__(self, dim: int, theta: float, max_position: int, scaling: Optional[dict] = None,
+                 precise: bool = False):
+        """``precise``: frequencies, angles, cosines and sines are worked out in 64-bit and rounded
+        once, so that a table row is the nearest float to the true value at any position."""
         if dim % 2:
             raise ValueError(f"rotary width {dim} must be even")
         self.rotary_dim = dim
@@ -60,19 +65,28 @@ class RotaryEncoding(PositionEncoding):
         self.max_position = max_position
         self.positions = max_position      # rows of the table: max_position, or fewer (``limit_positions``)
         self.scaling = scaling
+        self.precise = bool(precise)
         self.table: Optional[torch.Tensor] = None
 
     def limit_positions(self, n: int) -> None:
         self.positions = max(1, min(self.max_position, int(n)))
 
     def build_table(self) -> torch.Tensor:
+        if self.precise:
+            if self.scaling and self.scaling.get("rope_type", "default") not in ("default", "linear"):
+                raise ValueError("the 64-bit table knows plain and linearly scaled frequencies")
+            factor = float(self.scaling["factor"]) if self.scaling and self.scaling.get("rope_type") == "linear" else 1.0
+            idx = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64)
+            freq = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -idx / self.rotary_dim) / factor
+            angles = torch.outer(torch.arange(self.positions, dtype=torch.float64), freq)
+            return torch.cat((angles.cos(), angles.sin()), dim=-1).float().contiguous()
         inv_freq = rotary_inv_freq(self.rotary_dim, self.theta, self.scaling)
         angles = torch.outer(torch.arange(self.positions, dtype=torch.float32), inv_freq)
         return torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous()
 
     def materialize(self, device, dtype):
         scaling = tuple(sorted(self.scaling.items())) if self.scaling else None
-        key = (self.rotary_dim, self.theta, scaling, self.positions, str(torch.device(device)))
+        key = (self.rotary_dim, self.theta, scaling, self.positions, str(torch.device(device)), self.precise)
         table = _TABLES.get(key)
         if table is None:
             table = self.build_table().to(device)
