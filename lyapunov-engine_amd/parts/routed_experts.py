@@ -28,6 +28,9 @@ from .base import FeedForward, StepContext, WeightSource, WeightSpec
 class RoutedExperts(FeedForward):
     # ``forward`` takes the other branch's output as ``addend`` and returns the sum of both.
     takes_addend = True
+    # A list here receives every call's chosen experts (int32 [T, top], on the device), in the order
+    # of the calls: for load statistics, and for comparing a run with another that must route alike.
+    choices_log: Optional[list] = None
 
     def __init__(self, hidden_size: int, num_experts: int, top: int, intermediate_size: int, limit: float,
                  gate_slope: float = 1.702, shared_size: int = 0, shared_limit: float = 0.0,
@@ -75,6 +78,8 @@ class RoutedExperts(FeedForward):
         T = x.shape[0]
         logits = ops.linear(x, self.router_f, out_dtype=torch.float32)
         idx, wgt = ops.moe_route(logits, self.router_bias_f, self.top)
+        if RoutedExperts.choices_log is not None:
+            RoutedExperts.choices_log.append(idx)
         plan = ops.moe_sort(idx, self.num_experts)
         act = ops.moe_gemm(x, self.gate_up, plan, gated=True, limit=self.limit, alpha=self.gate_slope)
         y = ops.moe_gemm(act, self.down, plan, gated=False)

@@ -70,11 +70,15 @@ def attention(h: torch.Tensor, w: dict, m: dict, eps: float, positions: torch.Te
     q = rms_norm(h @ w["q"].T, w["q.norm"], eps).view(n, H, D)      # one norm over all heads' rows
     k = rms_norm(h @ w["k"].T, w["k.norm"], eps).view(n, G, D)
     v = (h @ w["v"].T).view(n, G, V)
-    rot = m["rot"]
-    factor = float(rot["scaling"]["factor"]) if rot.get("scaling") else 1.0
-    q = rotate_neighbours(q, pos, float(rot["base"]), int(rot["dims"]), factor)
-    k = rotate_neighbours(k, pos, float(rot["base"]), int(rot["dims"]), factor)
-    size, keep = int(m["mask"]["size"]), int(m["mask"]["keep_first"])
+    rot = m.get("rot")
+    if rot and int(rot["dims"]):                                    # no entry, or no dimensions: nothing turns
+        factor = float(rot["scaling"]["factor"]) if rot.get("scaling") else 1.0
+        q = rotate_neighbours(q, pos, float(rot["base"]), int(rot["dims"]), factor)
+        k = rotate_neighbours(k, pos, float(rot["base"]), int(rot["dims"]), factor)
+    if m.get("mask"):
+        size, keep = int(m["mask"]["size"]), int(m["mask"].get("keep_first", 0))
+    else:
+        size, keep = n + int(pos.max()) + 1, 0                      # no mask: every earlier token is seen
     mask = visible(pos, pos, size, keep)
     out = torch.zeros(n, H, V, dtype=h.dtype)
     for head in range(H):
@@ -92,18 +96,28 @@ def expert(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Te
     return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ down.T
 
 
-def route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor, top: int):
-    """-> (experts [n, top], weights [n, top]): the ``top`` largest of W_router h + bias, and the
-    softmax over those alone."""
+def route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor, top: int, chosen: torch.Tensor | None = None):
+    """-> (experts [n, top], weights [n, top], margin [n]): the ``top`` largest of W_router h + bias,
+    and the softmax over those alone; the margin is what the last chosen logit has over the first
+    one left out.  With ``chosen`` the choice is given (another run's, where the two must route
+    alike to be compared) and only the weights are worked out."""
     z = h @ router.T + bias
-    val, idx = torch.topk(z, top, dim=-1)
-    return idx, torch.softmax(val, dim=-1)
+    srt = torch.sort(z, dim=-1, descending=True).values
+    margin = srt[:, top - 1] - srt[:, top] if top < z.shape[1] else torch.full((z.shape[0],), float("inf"), dtype=z.dtype)
+    if chosen is None:
+        val, idx = torch.topk(z, top, dim=-1)
+    else:
+        idx = chosen.long()
+        val = torch.gather(z, 1, idx)
+    return idx, torch.softmax(val, dim=-1), margin
 
 
-def moe(h: torch.Tensor, w: dict, mlp: dict) -> torch.Tensor:
+def moe(h: torch.Tensor, w: dict, mlp: dict, chosen: torch.Tensor | None = None, notes: dict | None = None) -> torch.Tensor:
     """``w``: the feed-forward's tensors by short name (router, router.b, e<j>.gate/up/down,
-    shared.gate/up/down)."""
-    idx, wt = route(h, w["router"], w["router.b"], int(mlp["router"]["top"]))
+    shared.gate/up/down).  ``notes`` receives the choice and its margin."""
+    idx, wt, margin = route(h, w["router"], w["router.b"], int(mlp["router"]["top"]), chosen)
+    if notes is not None:
+        notes.update(chosen=idx, margin=margin)
     out = torch.zeros_like(h)
     limit = float(mlp["expert"]["limit"])
     for t in range(h.shape[0]):
@@ -119,12 +133,12 @@ def sub(tensors: dict, prefix: str) -> dict:
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def layer(x: torch.Tensor, tensors: dict, i: int, lc: dict, eps: float) -> torch.Tensor:
+def layer(x: torch.Tensor, tensors: dict, i: int, lc: dict, eps: float, chosen=None, notes=None) -> torch.Tensor:
     """x + mixer(n) + ff(n) with n = norm1(x)."""
     n = rms_norm(x, tensors[f"l{i}.norm1"], eps)
     y = attention(n, sub(tensors, f"l{i}.mix."), lc["mixer"], eps)
     if lc.get("mlp"):
-        y = y + moe(n, sub(tensors, f"l{i}.mlp."), lc["mlp"])
+        y = y + moe(n, sub(tensors, f"l{i}.mlp."), lc["mlp"], chosen, notes)
     return x + y
 
 
@@ -141,15 +155,25 @@ def running_order(cfg: dict) -> list:
     return order + [(i, False) for i in range(b, n)]
 
 
-def forward(cfg: dict, tensors: dict, tokens, collect: list | None = None) -> torch.Tensor:
-    """Logits [n, vocab] of one sequence; ``collect`` receives the stream after every layer run."""
+def forward(cfg: dict, tensors: dict, tokens, collect: list | None = None, chosen: list | None = None,
+            notes: list | None = None) -> torch.Tensor:
+    """Logits [n, vocab] of one sequence; ``collect`` receives the stream after every layer run.
+    ``chosen``: for every layer run with a routed feed-forward, in running order, the experts to use
+    [n, top]; ``notes`` receives a dict per such run (the choice made, its margin)."""
+    routed = 0
     eps = float(cfg["norm"]["eps"])
     x0 = tensors["embed"][torch.as_tensor(tokens, dtype=torch.long)]
     x = x0
     for i, again in running_order(cfg):
         if again:
             x = x + x0
-        x = layer(x, tensors, i, cfg["layers"][i], eps)
+        note = {} if notes is not None else None
+        has_ff = bool(cfg["layers"][i].get("mlp"))
+        x = layer(x, tensors, i, cfg["layers"][i], eps, chosen[routed] if chosen is not None and has_ff else None, note)
+        if has_ff:
+            routed += 1
+            if notes is not None:
+                notes.append(note)
         if collect is not None:
             collect.append(x.clone())
     return rms_norm(x, tensors["final.norm"], eps) @ tensors["embed"].T
