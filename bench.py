@@ -79,7 +79,32 @@ def faledra_shape(width, heads, ff, layers, vocab, q_rank, kv_rank):
                 layers=[gru() if i % 4 == 3 else latent() for i in range(layers)])
 
 
-# name -> (Faledra configuration, the Llama shape beside it); the looped stretch makes layers + 4 layer runs
+# Ronupel models likewise: attention layers of a real model's sizes with a window of 1,024 tokens that
+# keeps the first four, a sink, frequencies divided by 8; every layer routes a token to `top` of
+# `experts` experts and adds a shared one, the experts a token uses having together the width of the
+# Llama shape's feed-forward beside it; the first four layers run twice.
+def ronupel_shape(width, heads, kv_heads, dim, layers, vocab, experts, top, ff, shared):
+    def layer():
+        return dict(type="attention",
+                    mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5,
+                               mask=dict(size=1024, keep_first=4),
+                               rot=dict(base=500000.0, dims=dim // 2, scaling=dict(factor=8.0))),
+                    mlp=dict(kind="moe", router=dict(experts=experts, top=top), expert=dict(ff=ff, limit=7.0),
+                             shared=dict(ff=shared, limit=7.0)))
+
+    return dict(architecture="Ronupel", vocab=vocab, width=width, norm=dict(eps=1e-5),
+                loop=dict(start=0, stop=4, times=2), layers=[layer() for _ in range(layers)])
+
+
+# name -> (the design's configuration, the Llama shape beside it); the looped stretch makes layers + 4 layer runs
+RONUPEL_SIZES = {
+    "small": (ronupel_shape(1024, 16, 4, 64, 4, 32000, 16, 3, 1024, 1024),
+              dict(MODEL, vocab_size=32000, hidden_size=1024, intermediate_size=4096, num_hidden_layers=8,
+                   num_attention_heads=16, num_key_value_heads=4)),
+    "1b": (ronupel_shape(2048, 32, 8, 64, 12, 128256, 32, 4, 1536, 2048), dict(MODEL, num_hidden_layers=16)),
+    "wide": (ronupel_shape(4096, 32, 8, 128, 4, 128256, 32, 4, 3072, 2048),
+             dict(SHAPES["8b"], num_hidden_layers=8, head_dim=128)),
+}
 DESIGN_SIZES = {
     "small": (faledra_shape(1024, 16, 4096, 4, 32000, 384, 128),
               dict(MODEL, vocab_size=32000, hidden_size=1024, intermediate_size=4096, num_hidden_layers=8,
@@ -125,14 +150,16 @@ class _Vocab:
 
 
 def run_design(args):
-    """Prefill and decode speed of the Faledra sizes, each beside the Llama shape of equal size."""
+    """Prefill and decode speed of another design's sizes, each beside the Llama shape of equal size."""
     import torch
 
     context, block_size, out = 2304, 16, {}
-    for size in (args.size.split(",") if args.size else sorted(DESIGN_SIZES)):
-        faledra, llama = DESIGN_SIZES[size]
+    design = args.design
+    sizes = {"faledra": DESIGN_SIZES, "ronupel": RONUPEL_SIZES}[design]
+    for size in (args.size.split(",") if args.size else sorted(sizes)):
+        other, llama = sizes[size]
         out[size] = {}
-        for name, raw in (("faledra", faledra), ("llama", llama)):
+        for name, raw in ((design, other), ("llama", llama)):
             engine, _ = build_engine_from_config(raw, args.dtype, 8 * (context // block_size + 1) + 64 + 2048 // block_size,
                                                  8, block_size, budget=8192, max_model_len=context)
             cfg = _Vocab(engine)
@@ -151,12 +178,12 @@ def run_design(args):
             torch.cuda.empty_cache()
     first = out[sorted(out)[0]]
     print(json.dumps({
-        "metric": "Faledra beside the Llama shape of equal size: prefill and decode tok/s", "unit": "tok/s",
-        "value": first["faledra"]["decode_b8_ctx2048_tok_s"], "n_gpus": 1, "steps": min(args.steps, 64),
-        "warmup": min(args.warmup, 8), "ms_per_step": first["faledra"]["decode_b8_ms"], "higher_is_better": True,
+        "metric": f"{design.capitalize()} beside the Llama shape of equal size: prefill and decode tok/s", "unit": "tok/s",
+        "value": first[design]["decode_b8_ctx2048_tok_s"], "n_gpus": 1, "steps": min(args.steps, 64),
+        "warmup": min(args.warmup, 8), "ms_per_step": first[design]["decode_b8_ms"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic (random weights seed 4, random token ids)",
-        "config": {"model": "faledra", "sizes": sorted(out), "context_len": context, "kv_block_size": block_size,
+        "config": {"model": design, "sizes": sorted(out), "context_len": context, "kv_block_size": block_size,
                    "parallelism": "single-gpu", "graphs": True},
         "sizes": out}))
     return 0
@@ -371,15 +398,15 @@ def main():
                     help="mixed: the continuous batch of BASELINE.json configs[3] instead of the headline")
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode and the prefill")
     ap.add_argument("--skip-check", action="store_true", help="no comparison of bfloat16 logits with a 32-bit run")
-    ap.add_argument("--design", default="llama", choices=["llama", "faledra"],
-                    help="faledra: that design's prefill and decode speed at a few sizes, each beside the Llama "
-                         "shape of equal size, instead of the headline")
-    ap.add_argument("--size", default="", help="with --design faledra: which sizes, with commas (default: all)")
+    ap.add_argument("--design", default="llama", choices=["llama", "faledra", "ronupel"],
+                    help="faledra, ronupel: that design's prefill and decode speed at a few sizes, each beside the "
+                         "Llama shape of equal size, instead of the headline")
+    ap.add_argument("--size", default="", help="with another --design: which sizes, with commas (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
-    if args.design == "faledra":
+    if args.design != "llama":
         return run_design(args)
 
     import torch

@@ -30,18 +30,16 @@ constexpr int kRouteRegs = 8;            // experts per lane: up to 64 * 8 exper
 constexpr int kMostExperts = 64 * kRouteRegs;
 constexpr int kMostTop = 32;
 
-// z [rows, E] float logits without bias.  One wave per row.
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ bias,
-                                                        int rows, int E, int top, int32_t* __restrict__ idx,
-                                                        float* __restrict__ wgt) {
-  const int lane = threadIdx.x % kWave;
-  const int row = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  if (row >= rows) return;
+// One wave chooses for one row: z points at the row's E logits (bias not yet added).
+// `always` >= 0: one more pair is written after the chosen ones, expert `always` with weight 1 (an
+// expert every token uses, kept as one more matrix behind the routed ones).
+__device__ __forceinline__ void route_row(const float* z, const float* __restrict__ bias, int E, int top,
+                                          int32_t* __restrict__ idx, float* __restrict__ wgt, int lane, int always) {
   float v[kRouteRegs];
 #pragma unroll
   for (int r = 0; r < kRouteRegs; ++r) {
     const int e = lane + kWave * r;
-    v[r] = e < E ? z[static_cast<size_t>(row) * E + e] + (bias != nullptr ? bias[e] : 0.f) : LYP_NEG_INF;
+    v[r] = e < E ? z[e] + (bias != nullptr ? bias[e] : 0.f) : LYP_NEG_INF;
   }
   float chosen_v = 0.f;      // lane k keeps the k-th choice
   int chosen_e = 0;
@@ -66,8 +64,101 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   const float p = lane < top ? expf(chosen_v - m) : 0.f;
   const float total = wave_sum(p);
   if (lane < top) {
-    idx[static_cast<size_t>(row) * top + lane] = chosen_e;
-    wgt[static_cast<size_t>(row) * top + lane] = p / total;
+    idx[lane] = chosen_e;
+    wgt[lane] = p / total;
+  }
+  if (always >= 0 && lane == top) {
+    idx[top] = always;
+    wgt[top] = 1.0f;
+  }
+}
+
+// z [rows, E] float logits without bias.  One wave per row.
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ bias,
+                                                        int rows, int E, int top, int32_t* __restrict__ idx,
+                                                        float* __restrict__ wgt, int always) {
+  const int lane = threadIdx.x % kWave;
+  const int row = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (row >= rows) return;
+  const int per = top + (always >= 0 ? 1 : 0);
+  route_row(z + static_cast<size_t>(row) * E, bias, E, top, idx + static_cast<size_t>(row) * per,
+            wgt + static_cast<size_t>(row) * per, lane, always);
+}
+
+// The router's product and the choice in one kernel: x [rows, K] in T, the router's matrix
+// w [E, K] in float; logits in 32-bit on the float matrix instruction.  A workgroup takes 16 rows;
+// its four waves share the inner dimension (a quarter each, added up in the order of the waves), walk
+// the experts in blocks of 16, eight blocks a pass, and then choose for four rows each.
+constexpr int kRouteBlocks = 8;   // blocks of 16 experts whose sums a wave holds at a time
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_fused_kernel(const T* __restrict__ x, int ldx,
+                                                              const float* __restrict__ w,
+                                                              const float* __restrict__ bias, int rows, int E, int K,
+                                                              int top, int32_t* __restrict__ idx,
+                                                              float* __restrict__ wgt, int always) {
+  extern __shared__ float s_route[];                 // [4 waves][kRouteBlocks][64 lanes][4], then z [16][E]
+  float* s_part = s_route;
+  float* s_z = s_route + 4 * kRouteBlocks * kWave * 4;
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int t0 = blockIdx.x * 16;
+  const int r = lane % 16, grp = lane / 16;
+  const int row = t0 + r;
+  const T* xrow = x + static_cast<size_t>(min(row, rows - 1)) * ldx;
+  // this wave's share of the inner dimension, in steps of 16
+  const int steps = (K + 15) / 16;
+  const int s_begin = steps * wave / 4, s_end = steps * (wave + 1) / 4;
+  const int e_blocks = (E + 15) / 16;
+  for (int eb0 = 0; eb0 < e_blocks; eb0 += kRouteBlocks) {
+    f32x4 acc[kRouteBlocks];
+#pragma unroll
+    for (int b = 0; b < kRouteBlocks; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int st = s_begin; st < s_end; ++st) {
+      const int k = st * 16 + grp * 4;
+      f32x4 xf;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) xf[i] = (row < rows && k + i < K) ? to_f32(xrow[k + i]) : 0.f;
+#pragma unroll
+      for (int b = 0; b < kRouteBlocks; ++b) {
+        const int e = (eb0 + b) * 16 + r;
+        if ((eb0 + b) * 16 >= E) continue;
+        f32x4 wf;
+        const float* wrow = w + static_cast<size_t>(min(e, E - 1)) * K;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wf[i] = (e < E && k + i < K) ? wrow[k + i] : 0.f;
+        acc[b] = Mma16<float>::mma(wf, xf, acc[b]);     // acc[i]: row l % 16, expert block's 4 * (l / 16) + i
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < kRouteBlocks; ++b)
+      *reinterpret_cast<f32x4*>(&s_part[((wave * kRouteBlocks + b) * kWave + lane) * 4]) = acc[b];
+    __syncthreads();
+    // the four waves' shares added up in their order; thread -> (block, lane) pairs
+    for (int p = threadIdx.x; p < kRouteBlocks * kWave; p += 256) {
+      const int b = p / kWave, l = p % kWave;
+      if ((eb0 + b) * 16 >= E) continue;
+      f32x4 sum = *reinterpret_cast<const f32x4*>(&s_part[((0 * kRouteBlocks + b) * kWave + l) * 4]);
+#pragma unroll
+      for (int wv = 1; wv < 4; ++wv) {
+        const f32x4 o = *reinterpret_cast<const f32x4*>(&s_part[((wv * kRouteBlocks + b) * kWave + l) * 4]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sum[i] += o[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = (eb0 + b) * 16 + 4 * (l / 16) + i;
+        if (e < E) s_z[(l % 16) * E + e] = sum[i];
+      }
+    }
+    __syncthreads();
+  }
+  for (int q = wave; q < 16; q += 4) {
+    const int rr = t0 + q;
+    if (rr >= rows) break;
+    const int per = top + (always >= 0 ? 1 : 0);
+    route_row(s_z + q * E, bias, E, top, idx + static_cast<size_t>(rr) * per, wgt + static_cast<size_t>(rr) * per, lane,
+              always);
   }
 }
 
@@ -307,20 +398,45 @@ __global__ void glu_clamped_kernel(const T* __restrict__ gate_up, T* __restrict_
 }
 
 // out [rows, H] float = addend + shared + sum_k wgt[row, k] * y[place_of[row * top + k]]
+// One workgroup a row; the row's places and weights are read once, and every thread then has
+// several columns' loads in flight at a time.
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int32_t* __restrict__ place_of,
                                    const float* __restrict__ wgt, int top, const T* __restrict__ addend,
                                    const T* __restrict__ shared, float* __restrict__ out, int rows, int H) {
+  __shared__ int32_t s_at[kMostTop];
+  __shared__ float s_w[kMostTop];
   const int row = blockIdx.x;
-  for (int c = threadIdx.x; c < H; c += blockDim.x) {
-    float v = 0.f;
-    if (addend != nullptr) v += to_f32(addend[static_cast<size_t>(row) * H + c]);
-    if (shared != nullptr) v += to_f32(shared[static_cast<size_t>(row) * H + c]);
-    for (int k = 0; k < top; ++k) {
-      const int at = place_of[static_cast<size_t>(row) * top + k];
-      v += wgt[static_cast<size_t>(row) * top + k] * to_f32(y[static_cast<size_t>(at) * H + c]);
+  if (threadIdx.x < top) {
+    s_at[threadIdx.x] = place_of[static_cast<size_t>(row) * top + threadIdx.x];
+    s_w[threadIdx.x] = wgt[static_cast<size_t>(row) * top + threadIdx.x];
+  }
+  __syncthreads();
+  constexpr int U = 4;
+  for (int c0 = threadIdx.x; c0 < H; c0 += U * blockDim.x) {
+    float v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u * blockDim.x;
+      v[u] = 0.f;
+      if (c >= H) continue;
+      if (addend != nullptr) v[u] += to_f32(addend[static_cast<size_t>(row) * H + c]);
+      if (shared != nullptr) v[u] += to_f32(shared[static_cast<size_t>(row) * H + c]);
     }
-    out[static_cast<size_t>(row) * H + c] = v;
+    for (int k = 0; k < top; ++k) {
+      const size_t base = static_cast<size_t>(s_at[k]) * H;
+      const float wk = s_w[k];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int c = c0 + u * blockDim.x;
+        if (c < H) v[u] += wk * to_f32(y[base + c]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u * blockDim.x;
+      if (c < H) out[static_cast<size_t>(row) * H + c] = v[u];
+    }
   }
 }
 
@@ -332,13 +448,36 @@ extern "C" {
 
 int lyp_moe_most_experts() { return kMostExperts; }
 
-int lyp_moe_route(const float* z, const float* bias, int rows, int E, int top, int32_t* idx, float* wgt,
+int lyp_moe_route(const float* z, const float* bias, int rows, int E, int top, int32_t* idx, float* wgt, int always,
                   hipStream_t stream) {
   LYP_REQUIRE(rows >= 0 && E > 0 && E <= kMostExperts && top > 0 && top <= E && top <= kMostTop,
               "moe_route: %d rows, %d experts (at most %d), %d chosen (at most %d)", rows, E, kMostExperts, top,
               kMostTop);
   if (rows == 0) return 0;
-  moe_route_kernel<<<(rows + 3) / 4, 256, 0, stream>>>(z, bias, rows, E, top, idx, wgt);
+  LYP_REQUIRE(top < kMostTop || always < 0, "moe_route: %d chosen and one more", top);
+  moe_route_kernel<<<(rows + 3) / 4, 256, 0, stream>>>(z, bias, rows, E, top, idx, wgt, always);
+  LYP_LAUNCH_CHECK("moe_route");
+  return 0;
+}
+
+// x [rows, K] in the activations' type, w [E, K] float: the router's logits, the choice and the weights.
+int lyp_moe_route_fused(const void* x, int ldx, int dtype, const float* w, const float* bias, int rows, int E, int K,
+                        int top, int32_t* idx, float* wgt, int always, hipStream_t stream) {
+  LYP_REQUIRE(rows >= 0 && E > 0 && E <= kMostExperts && top > 0 && top <= E && top <= kMostTop && K > 0 && ldx >= K,
+              "moe_route: %d rows, %d experts (at most %d), %d chosen (at most %d), inner size %d", rows, E,
+              kMostExperts, top, kMostTop, K);
+  LYP_REQUIRE(top < kMostTop || always < 0, "moe_route: %d chosen and one more", top);
+  if (rows == 0) return 0;
+  const size_t lds = sizeof(float) * (4 * kRouteBlocks * kWave * 4 + 16 * E);
+  const int blocks = (rows + 15) / 16;
+  if (dtype == kF32)
+    moe_route_fused_kernel<float><<<blocks, 256, lds, stream>>>(static_cast<const float*>(x), ldx, w, bias, rows, E, K,
+                                                                top, idx, wgt, always);
+  else if (dtype == kBF16)
+    moe_route_fused_kernel<bf16_t><<<blocks, 256, lds, stream>>>(static_cast<const bf16_t*>(x), ldx, w, bias, rows, E,
+                                                                 K, top, idx, wgt, always);
+  else
+    LYP_REQUIRE(false, "moe_route: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("moe_route");
   return 0;
 }
@@ -423,7 +562,8 @@ int lyp_moe_combine(const void* y, const int32_t* place_of, const float* wgt, in
                     const void* shared, float* out, int dtype, int rows, int H, hipStream_t stream) {
   LYP_REQUIRE(rows >= 0 && H > 0 && top > 0, "moe_combine: bad sizes");
   if (rows == 0) return 0;
-  const int threads = H >= 1024 ? 256 : 128;
+  LYP_REQUIRE(top <= kMostTop, "moe_combine: %d choices a token (at most %d)", top, kMostTop);
+  const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 128);
   if (dtype == kF32)
     moe_combine_kernel<float><<<rows, threads, 0, stream>>>(static_cast<const float*>(y), place_of, wgt, top,
                                                             static_cast<const float*>(addend),

@@ -113,7 +113,9 @@ def core() -> ctypes.CDLL:
                                       c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p, c_int, c_int, c_int,
                                       c_int, c_int, c_int, c_int, c_void_p]
         lib.lyp_stream_add.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_longlong, c_void_p]
-        lib.lyp_moe_route.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+        lib.lyp_moe_route.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]
+        lib.lyp_moe_route_fused.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                            c_void_p, c_void_p, c_int, c_void_p]
         lib.lyp_moe_tile_rows.argtypes = [c_int, c_int]
         lib.lyp_moe_most_tiles.argtypes = [c_int, c_int, c_int]
         lib.lyp_moe_sort.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -1345,16 +1347,36 @@ def glu_clamped(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tens
     return out
 
 
-def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, top: int):
+def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, top: int, always: int = -1):
     """float router logits [T, E] (+ bias) -> (experts int32 [T, top], weights float [T, top]): the
-    ``top`` largest (of equal ones the first) and the softmax over those alone."""
+    ``top`` largest (of equal ones the first) and the softmax over those alone.  ``always`` >= 0: one
+    more pair a token, that expert with weight 1 (results are [T, top + 1])."""
     _dev(logits, bias)
     _f32(logits, bias)
     T, E = logits.shape
-    idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
-    wgt = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    per = top + (1 if always >= 0 else 0)
+    idx = torch.empty((T, per), dtype=torch.int32, device=logits.device)
+    wgt = torch.empty((T, per), dtype=torch.float32, device=logits.device)
     lib = core()
-    _check(lib.lyp_moe_route(_p(logits), _p(bias), T, E, top, _p(idx), _p(wgt), _stream()), lib)
+    _check(lib.lyp_moe_route(_p(logits), _p(bias), T, E, top, _p(idx), _p(wgt), int(always), _stream()), lib)
+    return idx, wgt
+
+
+def moe_route_from(x: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, top: int, always: int = -1):
+    """As ``moe_route`` from the router's input: x [T, K] activations, ``router`` [E, K] float; the
+    logits x @ router.T are formed in 32-bit in the same kernel."""
+    _dev(x, router, bias)
+    _f32(router, bias)
+    T, K = x.shape
+    E = router.shape[0]
+    if router.shape[1] != K or x.stride(1) != 1:
+        raise KernelError(f"moe_route_from: x {tuple(x.shape)}, router {tuple(router.shape)}")
+    per = top + (1 if always >= 0 else 0)
+    idx = torch.empty((T, per), dtype=torch.int32, device=x.device)
+    wgt = torch.empty((T, per), dtype=torch.float32, device=x.device)
+    lib = core()
+    _check(lib.lyp_moe_route_fused(_p(x), x.stride(0), _code(x.dtype), _p(router), _p(bias), T, E, K, top, _p(idx),
+                                   _p(wgt), int(always), _stream()), lib)
     return idx, wgt
 
 

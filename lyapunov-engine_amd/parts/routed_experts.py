@@ -44,6 +44,9 @@ class RoutedExperts(FeedForward):
                  down="down")
         n.update(names or {})
         self.names = n
+        # A shared expert of the routed experts' size and limit is kept as one more matrix behind
+        # theirs and rides in their products as an expert every token uses with weight 1.
+        self.shared_folded = self.shared_size == self.intermediate_size and self.shared_limit == self.limit
         self.router = self.router_bias = self.gate_up = self.down = self.shared_gate_up = self.shared_down = None
         self.router_f = self.router_bias_f = None
 
@@ -54,10 +57,14 @@ class RoutedExperts(FeedForward):
             e = n["expert"].format(j=j)
             gate_up += [WeightSource(e + n["gate"], (I, H)), WeightSource(e + n["up"], (I, H))]
             down.append(WeightSource(e + n["down"], (H, I)))
+        if self.shared_folded:
+            s = n["shared"]
+            gate_up += [WeightSource(s + n["gate"], (I, H)), WeightSource(s + n["up"], (I, H))]
+            down.append(WeightSource(s + n["down"], (H, I)))
         specs = [WeightSpec("router", (WeightSource(n["router"], (E, H)),)),
                  WeightSpec("router_bias", (WeightSource(n["router_bias"], (E,)),)),
                  WeightSpec("gate_up", tuple(gate_up)), WeightSpec("down", tuple(down))]
-        if self.shared_size:
+        if self.shared_size and not self.shared_folded:
             s, S = n["shared"], self.shared_size
             specs += [WeightSpec("shared_gate_up", (WeightSource(s + n["gate"], (S, H)), WeightSource(s + n["up"], (S, H)))),
                       WeightSpec("shared_down", (WeightSource(s + n["down"], (H, S)),))]
@@ -69,22 +76,23 @@ class RoutedExperts(FeedForward):
         self.router_f = self.router.float().contiguous()
         self.router_bias_f = self.router_bias.float().contiguous()
         self.router = None
-        self.gate_up = self.gate_up.view(E, 2 * I, H)      # per expert: gate rows, then up rows
-        self.down = self.down.view(E, H, I)
+        stacked = E + (1 if self.shared_folded else 0)
+        self.gate_up = self.gate_up.view(stacked, 2 * I, H)      # per expert: gate rows, then up rows
+        self.down = self.down.view(stacked, H, I)
 
     def forward(self, ctx: StepContext, x, addend=None):
         """-> float [1, T, hidden] (one slice of partial sums): the experts' weighted outputs, the
         shared expert's and ``addend`` (the other branch's output, activations [T, hidden])."""
         T = x.shape[0]
-        logits = ops.linear(x, self.router_f, out_dtype=torch.float32)
-        idx, wgt = ops.moe_route(logits, self.router_bias_f, self.top)
+        always = self.num_experts if self.shared_folded else -1
+        idx, wgt = ops.moe_route_from(x, self.router_f, self.router_bias_f, self.top, always)
         if RoutedExperts.choices_log is not None:
-            RoutedExperts.choices_log.append(idx)
-        plan = ops.moe_sort(idx, self.num_experts)
+            RoutedExperts.choices_log.append(idx[:, :self.top])
+        plan = ops.moe_sort(idx, self.gate_up.shape[0])
         act = ops.moe_gemm(x, self.gate_up, plan, gated=True, limit=self.limit, alpha=self.gate_slope)
         y = ops.moe_gemm(act, self.down, plan, gated=False)
         shared = None
-        if self.shared_size:
+        if self.shared_size and not self.shared_folded:
             gu = ops.linear(x, self.shared_gate_up, out_dtype=ctx.dtype)
             shared = ops.linear(ops.glu_clamped(gu, self.shared_limit, self.gate_slope), self.shared_down,
                                 out_dtype=ctx.dtype)

@@ -20,6 +20,9 @@ import collections
 import sqlite3
 
 
+LONGEST = 10 ** 9      # ``--step`` value for "the step that took longest" (a prompt among decode steps)
+
+
 def short(name: str) -> str:
     for mark in ("lyp::", "_ZN3lyp"):
         i = name.find(mark)
@@ -33,7 +36,11 @@ def summarise(db: str, step: int) -> str:
     con = sqlite3.connect(db)
     rows = con.execute(
         "select name, start, end, grid_x, grid_y, grid_z, workgroup_x from kernels order by start").fetchall()
-    starts = [i for i, r in enumerate(rows) if "embedding_kernel" in r[0]]
+    # (a model that adds the embedding's output again later in the step looks it up twice in a row)
+    starts = [i for i, r in enumerate(rows) if "embedding_kernel" in r[0] and (i == 0 or "embedding_kernel" not in rows[i - 1][0])]
+    if step == LONGEST:
+        ends = starts[1:] + [len(rows)]
+        step = max(range(len(starts)), key=lambda k: rows[ends[k] - 1][2] - rows[starts[k]][1])
     if len(starts) < 2:
         raise SystemExit("the trace holds fewer than two engine steps")
     a = starts[step]
@@ -73,11 +80,12 @@ def main() -> None:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("db", help="rocprofv3's NAME_results.db")
     ap.add_argument("--step", type=int, default=-3, help="which step (negative: from the end)")
+    ap.add_argument("--longest", action="store_true", help="the step that took longest instead")
     ap.add_argument("--all", action="store_true", help="every kernel of the trace by name and shape (a program that "
                     "is no engine: kernel_bench), not one engine step")
     ap.add_argument("--skip", type=int, default=2, help="with --all: launches of every kind left out as warm-up")
     args = ap.parse_args()
-    print(summarise_all(args.db, args.skip) if args.all else summarise(args.db, args.step))
+    print(summarise_all(args.db, args.skip) if args.all else summarise(args.db, LONGEST if args.longest else args.step))
 
 
 if __name__ == "__main__":

@@ -60,7 +60,7 @@ CONFIGS = {
                                mlp=moe(16, 4, 24, 50.0, shared=(40, 0.3))),
                           attn(6, 3, 16, 16, dims=0, scale=0.5, mlp=moe(4, 2, 56, 0.2)),
                           attn(3, 3, 32, 32, window=64, keep=16, dims=8, base=77.0, factor=16.0, scale=0.3,
-                               mlp=moe(9, 3, 32, 1.0, shared=(16, 2.0)))],
+                               mlp=moe(9, 3, 32, 1.0, shared=(32, 1.0)))],      # a shared expert like the routed ones
                 loop=(1, 2, 3), eps=1e-6),
 }
 BLOCK_SIZE = {"A": 4, "B": 16, "C": 16}

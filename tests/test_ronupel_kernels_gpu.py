@@ -334,6 +334,33 @@ def test_router_chooses_the_largest_and_weighs_them_alone(sizes):
     assert float((wgt.sum(-1) - 1).abs().max()) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("sizes", [(5, 2, 72), (12, 3, 192), (64, 8, 100), (130, 4, 256), (300, 1, 64), (1, 1, 40)])
+def test_router_product_and_choice_in_one_kernel(dtype, sizes):
+    """Logits in 32-bit from the activations, then the choice, for 1, 16, 17 and many rows; one
+    more expert that every token uses may be appended with weight 1."""
+    from lyapunov_engine_amd.kernels import ops
+
+    E, top, K = sizes
+    g = torch.Generator().manual_seed(E + K)
+    w = torch.randn(E, K, generator=g)
+    bias = torch.randn(E, generator=g)
+    for T in (1, 16, 17, 700):
+        x = torch.randn(T, K, generator=g).to(tdt(dtype))
+        z = x.double() @ w.double().T + bias.double()
+        val, want_idx = torch.topk(z, top, dim=-1)
+        srt = torch.sort(z, -1, descending=True).values
+        clear = torch.ones(T, dtype=torch.bool) if top == E else (srt[:, top - 1] - srt[:, top]) > 1e-3
+        gaps = (srt[:, :top - 1] - srt[:, 1:top]).min(-1).values if top > 1 else torch.ones(T)
+        clear &= gaps > 1e-3                                   # the order among the chosen, too
+        for always in (-1, E):
+            idx, wgt = ops.moe_route_from(x.to(DEV), w.to(DEV), bias.to(DEV), top, always)
+            assert torch.equal(idx.cpu().long()[clear][:, :top], want_idx[clear]), f"{T} rows"
+            close(wgt[:, :top][clear.to(DEV)], torch.softmax(val, -1)[clear], "float32", "weights", tol=1e-4)
+            if always >= 0:
+                assert (idx[:, top] == E).all() and (wgt[:, top] == 1.0).all()
+
+
 @pytest.mark.parametrize("shape", [(1, 1, 1), (7, 5, 2), (300, 12, 3), (2000, 8, 8), (1500, 70, 5), (1030, 3, 1)])
 def test_pairs_sorted_by_expert_in_their_own_order(shape):
     from lyapunov_engine_amd.kernels import ops
@@ -362,16 +389,20 @@ def test_pairs_sorted_by_expert_in_their_own_order(shape):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(1, 5, 2, 72, 40, 28), (7, 5, 2, 72, 40, 0), (300, 3, 3, 64, 20, 16), (40, 70, 5, 48, 8, 24),
-                                   (700, 4, 1, 100, 52, 0), (33, 16, 4, 192, 96, 64)])
+                                   (700, 4, 1, 100, 52, 0), (33, 16, 4, 192, 96, 64), (9, 6, 2, 64, 48, 48),
+                                   (900, 6, 2, 64, 48, 48), (70, 130, 3, 40, 16, 0)])
 def test_routed_experts_against_the_plain_mixture(dtype, shape):
     """The whole feed-forward part, with another branch's output added in, for steps of one token,
-    of few and of many (tiles of 16 and of 64 rows), sizes without 16-byte rows among them."""
+    of few and of many (tiles of 16 and of 64 rows), sizes without 16-byte rows among them, and a
+    shared expert of the routed experts' size and limit (it then rides in their products)."""
     from lyapunov_engine_amd.parts.base import StepContext
     from lyapunov_engine_amd.parts.routed_experts import RoutedExperts
 
     T, E, top, H, I, S = shape
     g = torch.Generator().manual_seed(T + E)
-    part = RoutedExperts(H, E, top, I, limit=1.2, gate_slope=1.702, shared_size=S, shared_limit=0.8)
+    shared_limit = 1.2 if S == I else 0.8
+    part = RoutedExperts(H, E, top, I, limit=1.2, gate_slope=1.702, shared_size=S, shared_limit=shared_limit)
+    assert part.shared_folded == (S == I)
     w = {}
     for ws in part.weight_specs():
         pieces = []
@@ -387,7 +418,7 @@ def test_routed_experts_against_the_plain_mixture(dtype, shape):
                       ctx_len=None, state_slots=None, logit_rows=None, R=0, groups=[])
     got = part.forward(ctx, x.to(DEV), addend=addend.to(DEV))
     assert got.dtype == torch.float32 and tuple(got.shape) == (1, T, H)
-    mlp = dict(router=dict(experts=E, top=top), expert=dict(ff=I, limit=1.2), shared=dict(ff=S, limit=0.8) if S else None)
+    mlp = dict(router=dict(experts=E, top=top), expert=dict(ff=I, limit=1.2), shared=dict(ff=S, limit=shared_limit) if S else None)
     wd = {k: v.double() for k, v in w.items()}
     want = RP.moe(x.double(), wd, mlp) + addend.double()
     # a router decision that hangs on rounding is no fault: leave such tokens out
