@@ -33,13 +33,28 @@ constexpr int kMostTop = 32;
 // One wave chooses for one row: z points at the row's E logits (bias not yet added).
 // `always` >= 0: one more pair is written after the chosen ones, expert `always` with weight 1 (an
 // expert every token uses, kept as one more matrix behind the routed ones).
+// `parts` > 1: the logits are the sum of that many partial sums, `part_stride` floats apart.
 __device__ __forceinline__ void route_row(const float* z, const float* __restrict__ bias, int E, int top,
-                                          int32_t* __restrict__ idx, float* __restrict__ wgt, int lane, int always) {
+                                          int32_t* __restrict__ idx, float* __restrict__ wgt, int lane, int always,
+                                          int parts = 1, size_t part_stride = 0) {
   float v[kRouteRegs];
 #pragma unroll
   for (int r = 0; r < kRouteRegs; ++r) {
     const int e = lane + kWave * r;
-    v[r] = e < E ? z[e] + (bias != nullptr ? bias[e] : 0.f) : LYP_NEG_INF;
+    if (e < E) {
+      // four partial sums asked for at a time, added in their order
+      float sum = 0.f;
+      for (int p0 = 0; p0 < parts; p0 += 4) {
+        float t[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) t[i] = p0 + i < parts ? z[(p0 + i) * part_stride + e] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sum += t[i];
+      }
+      v[r] = sum + (bias != nullptr ? bias[e] : 0.f);
+    } else {
+      v[r] = LYP_NEG_INF;
+    }
   }
   float chosen_v = 0.f;      // lane k keeps the k-th choice
   int chosen_e = 0;
@@ -76,30 +91,33 @@ __device__ __forceinline__ void route_row(const float* z, const float* __restric
 // z [rows, E] float logits without bias.  One wave per row.
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ bias,
                                                         int rows, int E, int top, int32_t* __restrict__ idx,
-                                                        float* __restrict__ wgt, int always) {
+                                                        float* __restrict__ wgt, int always, int parts) {
   const int lane = threadIdx.x % kWave;
   const int row = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
   if (row >= rows) return;
   const int per = top + (always >= 0 ? 1 : 0);
   route_row(z + static_cast<size_t>(row) * E, bias, E, top, idx + static_cast<size_t>(row) * per,
-            wgt + static_cast<size_t>(row) * per, lane, always);
+            wgt + static_cast<size_t>(row) * per, lane, always, parts, static_cast<size_t>(rows) * E);
 }
 
 // The router's product and the choice in one kernel: x [rows, K] in T, the router's matrix
 // w [E, K] in float; logits in 32-bit on the float matrix instruction.  A workgroup takes 16 rows;
-// its four waves share the inner dimension (a quarter each, added up in the order of the waves), walk
-// the experts in blocks of 16, eight blocks a pass, and then choose for four rows each.
-constexpr int kRouteBlocks = 8;   // blocks of 16 experts whose sums a wave holds at a time
+// its eight waves share the inner dimension (an eighth each, added up in the order of the waves),
+// walk the experts in blocks of 16, four blocks a pass, and then choose for two rows each.  A wave
+// asks for four steps' operands at once: the kernel is as long as its chain of loads.
+constexpr int kRouteBlocks = 4;   // blocks of 16 experts whose sums a wave holds at a time
+constexpr int kRouteWaves = 8;
+constexpr int kRouteAhead = 4;    // steps of 16 inner values whose loads are in flight together
 
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_fused_kernel(const T* __restrict__ x, int ldx,
-                                                              const float* __restrict__ w,
-                                                              const float* __restrict__ bias, int rows, int E, int K,
-                                                              int top, int32_t* __restrict__ idx,
-                                                              float* __restrict__ wgt, int always) {
-  extern __shared__ float s_route[];                 // [4 waves][kRouteBlocks][64 lanes][4], then z [16][E]
+__global__ __launch_bounds__(kRouteWaves* kWave) void moe_route_fused_kernel(
+    const T* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ bias, int rows, int E,
+    int K, int top, int32_t* __restrict__ idx, float* __restrict__ wgt, int always, int vec_ok,
+    float* __restrict__ part) {
+  extern __shared__ float s_route[];                 // [waves][kRouteBlocks][64 lanes][4], then z [16][E]
   float* s_part = s_route;
-  float* s_z = s_route + 4 * kRouteBlocks * kWave * 4;
+  float* s_z = s_route + kRouteWaves * kRouteBlocks * kWave * 4;
+  typedef T XVec __attribute__((ext_vector_type(4)));
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int t0 = blockIdx.x * 16;
@@ -107,40 +125,76 @@ __global__ __launch_bounds__(256) void moe_route_fused_kernel(const T* __restric
   const int row = t0 + r;
   const T* xrow = x + static_cast<size_t>(min(row, rows - 1)) * ldx;
   // this wave's share of the inner dimension, in steps of 16
+  // (grid y > 1: the workgroups of a row block share the inner dimension too, each leaves its sums in
+  // `part` [y][rows][E], and moe_route_kernel adds them up and chooses)
   const int steps = (K + 15) / 16;
-  const int s_begin = steps * wave / 4, s_end = steps * (wave + 1) / 4;
+  const int ks = gridDim.y, ky = blockIdx.y;
+  const int wg_begin = steps * ky / ks, wg_steps = steps * (ky + 1) / ks - wg_begin;
+  const int s_begin = wg_begin + wg_steps * wave / kRouteWaves, s_end = wg_begin + wg_steps * (wave + 1) / kRouteWaves;
   const int e_blocks = (E + 15) / 16;
+  auto load_x = [&](int st) {
+    const int k = st * 16 + grp * 4;
+    f32x4 xf = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (row < rows) {
+      if (vec_ok && k + 4 <= K) {
+        const XVec v = *reinterpret_cast<const XVec*>(xrow + k);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xf[i] = to_f32(v[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (k + i < K) xf[i] = to_f32(xrow[k + i]);
+      }
+    }
+    return xf;
+  };
+  auto load_w = [&](int st, int eb) {
+    const int k = st * 16 + grp * 4;
+    const int e = eb * 16 + r;
+    f32x4 wf = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (e < E) {
+      const float* wrow = w + static_cast<size_t>(e) * K;
+      if (vec_ok && k + 4 <= K) {
+        wf = *reinterpret_cast<const f32x4*>(wrow + k);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (k + i < K) wf[i] = wrow[k + i];
+      }
+    }
+    return wf;
+  };
   for (int eb0 = 0; eb0 < e_blocks; eb0 += kRouteBlocks) {
     f32x4 acc[kRouteBlocks];
 #pragma unroll
     for (int b = 0; b < kRouteBlocks; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int st = s_begin; st < s_end; ++st) {
-      const int k = st * 16 + grp * 4;
-      f32x4 xf;
+    for (int st0 = s_begin; st0 < s_end; st0 += kRouteAhead) {
+      f32x4 xf[kRouteAhead], wf[kRouteAhead][kRouteBlocks];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) xf[i] = (row < rows && k + i < K) ? to_f32(xrow[k + i]) : 0.f;
+      for (int a = 0; a < kRouteAhead; ++a) {
+        const int st = st0 + a;
+        xf[a] = st < s_end ? load_x(st) : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int b = 0; b < kRouteBlocks; ++b) {
-        const int e = (eb0 + b) * 16 + r;
-        if ((eb0 + b) * 16 >= E) continue;
-        f32x4 wf;
-        const float* wrow = w + static_cast<size_t>(min(e, E - 1)) * K;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) wf[i] = (e < E && k + i < K) ? wrow[k + i] : 0.f;
-        acc[b] = Mma16<float>::mma(wf, xf, acc[b]);     // acc[i]: row l % 16, expert block's 4 * (l / 16) + i
+        for (int b = 0; b < kRouteBlocks; ++b)
+          wf[a][b] = (st < s_end && eb0 + b < e_blocks) ? load_w(st, eb0 + b) : f32x4{0.f, 0.f, 0.f, 0.f};
       }
+#pragma unroll
+      for (int a = 0; a < kRouteAhead; ++a)
+#pragma unroll
+        for (int b = 0; b < kRouteBlocks; ++b)
+          acc[b] = Mma16<float>::mma(wf[a][b], xf[a], acc[b]);   // acc[i]: row l % 16, the block's expert 4 * (l / 16) + i
     }
 #pragma unroll
     for (int b = 0; b < kRouteBlocks; ++b)
       *reinterpret_cast<f32x4*>(&s_part[((wave * kRouteBlocks + b) * kWave + lane) * 4]) = acc[b];
     __syncthreads();
-    // the four waves' shares added up in their order; thread -> (block, lane) pairs
-    for (int p = threadIdx.x; p < kRouteBlocks * kWave; p += 256) {
+    // the waves' shares added up in their order; thread -> (block, lane)
+    for (int p = threadIdx.x; p < kRouteBlocks * kWave; p += kRouteWaves * kWave) {
       const int b = p / kWave, l = p % kWave;
-      if ((eb0 + b) * 16 >= E) continue;
-      f32x4 sum = *reinterpret_cast<const f32x4*>(&s_part[((0 * kRouteBlocks + b) * kWave + l) * 4]);
+      if (eb0 + b >= e_blocks) continue;
+      f32x4 sum = *reinterpret_cast<const f32x4*>(&s_part[(b * kWave + l) * 4]);
 #pragma unroll
-      for (int wv = 1; wv < 4; ++wv) {
+      for (int wv = 1; wv < kRouteWaves; ++wv) {
         const f32x4 o = *reinterpret_cast<const f32x4*>(&s_part[((wv * kRouteBlocks + b) * kWave + l) * 4]);
 #pragma unroll
         for (int i = 0; i < 4; ++i) sum[i] += o[i];
@@ -153,10 +207,17 @@ __global__ __launch_bounds__(256) void moe_route_fused_kernel(const T* __restric
     }
     __syncthreads();
   }
-  for (int q = wave; q < 16; q += 4) {
+  if (ks > 1) {
+    for (int i = threadIdx.x; i < 16 * E; i += kRouteWaves * kWave) {
+      const int rr = t0 + i / E;
+      if (rr < rows) part[(static_cast<size_t>(ky) * rows + rr) * E + i % E] = s_z[i];
+    }
+    return;
+  }
+  const int per = top + (always >= 0 ? 1 : 0);
+  for (int q = wave; q < 16; q += kRouteWaves) {
     const int rr = t0 + q;
     if (rr >= rows) break;
-    const int per = top + (always >= 0 ? 1 : 0);
     route_row(s_z + q * E, bias, E, top, idx + static_cast<size_t>(rr) * per, wgt + static_cast<size_t>(rr) * per, lane,
               always);
   }
@@ -244,7 +305,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
     int vec_ok) {
   using MW = Mma16Wide<T>;
   constexpr int VEC = 16 / sizeof(T);
-  constexpr int KT = 32;
+  constexpr int KT = 128 / sizeof(T);                 // inner values a round: 128 bytes of every row
   constexpr int LD = KT + (sizeof(T) == 2 ? 8 : 4);   // padded row: 16-byte reads of 16 rows fall into distinct banks
   constexpr int TM = 16 * MB, TN = 64;
   constexpr int BROWS = GATED ? 2 * TN : TN;
@@ -252,8 +313,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
   constexpr int STEPS = KT / (4 * MW::kElems);
   constexpr int A_PER = (TM * KT / VEC + 255) / 256, B_PER = (BROWS * KT / VEC + 255) / 256;
   typedef T VecT __attribute__((ext_vector_type(VEC)));
-  __shared__ __attribute__((aligned(16))) T As[TM * LD];
-  __shared__ __attribute__((aligned(16))) T Bs[BROWS * LD];
+  // two buffers: the next round's tiles are written while this round's are read, one barrier a round
+  __shared__ __attribute__((aligned(16))) T As2[2][TM * LD];
+  __shared__ __attribute__((aligned(16))) T Bs2[2][BROWS * LD];
 
   const int tile = blockIdx.x;
   if (tile >= n_tiles[0]) return;
@@ -319,13 +381,13 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
 #pragma unroll
     for (int n = 0; n < B_PER; ++n) b_reg[n] = fetch(b_src[n], k0 + b_k[n]);
   };
-  auto stash = [&] {
+  auto stash = [&](int buf) {
 #pragma unroll
     for (int n = 0; n < A_PER; ++n)
-      if (a_lds[n] >= 0) *reinterpret_cast<VecT*>(As + a_lds[n]) = a_reg[n];
+      if (a_lds[n] >= 0) *reinterpret_cast<VecT*>(As2[buf] + a_lds[n]) = a_reg[n];
 #pragma unroll
     for (int n = 0; n < B_PER; ++n)
-      if (b_lds[n] >= 0) *reinterpret_cast<VecT*>(Bs + b_lds[n]) = b_reg[n];
+      if (b_lds[n] >= 0) *reinterpret_cast<VecT*>(Bs2[buf] + b_lds[n]) = b_reg[n];
   };
 
   f32x4 acc[CB], acc_up[GATED ? CB : 1];
@@ -335,11 +397,14 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
   for (int c = 0; c < (GATED ? CB : 1); ++c) acc_up[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   load(0);
-  stash();
+  stash(0);
   __syncthreads();
+  int buf = 0;
   for (int k0 = 0; k0 < K; k0 += KT) {
     const bool more = k0 + KT < K;
     if (more) load(k0 + KT);
+    const T* As = As2[buf];
+    const T* Bs = Bs2[buf];
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       const int kk = s * 4 * MW::kElems + (lane / 16) * MW::kElems;
@@ -355,11 +420,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
         }
       }
     }
+    if (more) stash(buf ^ 1);
     __syncthreads();
-    if (more) {
-      stash();
-      __syncthreads();
-    }
+    buf ^= 1;
   }
 
   // lane l: token row wm * 16 + l % 16, features (wn * CB + c) * 16 + 4 * (l / 16) + {0..3}
@@ -379,6 +442,151 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
         y = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
       }
       orow[col + i] = from_f32<TO>(y);
+    }
+  }
+}
+
+// The same product for many rows an expert: tiles of 128 rows and 128 matrix rows (GATED: 64 gate
+// columns and their 64 up columns), four waves in 2 x 2, a wave 64 rows x 2 blocks of 32 matrix
+// rows on the 32x32 instruction, so that a fragment read from LDS feeds two products.
+template <typename T, bool GATED>
+__global__ __launch_bounds__(256) void moe_gemm_wide_kernel(
+    const T* __restrict__ a, int lda, const T* __restrict__ w, long long w_expert_stride, int ldw,
+    T* __restrict__ out, int ldo, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
+    const int32_t* __restrict__ n_tiles, const int32_t* __restrict__ expert_off,
+    const int32_t* __restrict__ sorted_pair, int top, int N, int K, int up_offset, float limit, float alpha,
+    int vec_ok) {
+  using MW = Mma32<T>;
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int KT = 64 / sizeof(T);                  // inner values a round
+  constexpr int LD = KT + (sizeof(T) == 2 ? 8 : 4);
+  constexpr int TM = 128, BROWS = 128;
+  constexpr int TN = GATED ? 64 : 128;                // output columns a workgroup
+  constexpr int STEPS = KT / (2 * MW::kElems);
+  constexpr int PER = TM * KT / VEC / 256;            // 16-byte pieces of a tile per thread (2)
+  typedef T VecT __attribute__((ext_vector_type(VEC)));
+  __shared__ __attribute__((aligned(16))) T As2[2][TM * LD];
+  __shared__ __attribute__((aligned(16))) T Bs2[2][BROWS * LD];
+
+  const int tile = blockIdx.x;
+  if (tile >= n_tiles[0]) return;
+  const int e = tile_expert[tile];
+  const int row0 = tile_row0[tile];
+  const int row_end = expert_off[e + 1];
+  const int c0 = blockIdx.y * TN;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave % 2, wn = wave / 2;
+  const T* we = w + static_cast<size_t>(e) * w_expert_stride;
+
+  const T* a_src[PER];
+  const T* b_src[PER];
+  int t_k[PER], t_lds[PER];
+#pragma unroll
+  for (int n = 0; n < PER; ++n) {
+    const int v = tid + n * 256;
+    const int r = v / (KT / VEC), kc = (v % (KT / VEC)) * VEC;
+    t_k[n] = kc;
+    t_lds[n] = r * LD + kc;
+    a_src[n] = nullptr;
+    if (row0 + r < row_end) {
+      const int place = row0 + r;
+      a_src[n] = a + static_cast<size_t>(GATED ? sorted_pair[place] / top : place) * lda;
+    }
+    // matrix rows of the tile: GATED: 64 gate rows, then the 64 up rows that go with them
+    const int col = GATED ? c0 + r % 64 : c0 + r;
+    b_src[n] = col < N ? we + static_cast<size_t>(col + (GATED && r >= 64 ? up_offset : 0)) * ldw : nullptr;
+  }
+  auto fetch = [&](const T* src, int k) {
+    VecT x;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) x[i] = from_f32<T>(0.f);
+    if (src != nullptr) {
+      if (vec_ok && k + VEC <= K) {
+        x = *reinterpret_cast<const VecT*>(src + k);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+          if (k + i < K) x[i] = src[k + i];
+      }
+    }
+    return x;
+  };
+  VecT a_reg[PER], b_reg[PER];
+  auto load = [&](int k0) {
+#pragma unroll
+    for (int n = 0; n < PER; ++n) {
+      a_reg[n] = fetch(a_src[n], k0 + t_k[n]);
+      b_reg[n] = fetch(b_src[n], k0 + t_k[n]);
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int n = 0; n < PER; ++n) {
+      *reinterpret_cast<VecT*>(As2[buf] + t_lds[n]) = a_reg[n];
+      *reinterpret_cast<VecT*>(Bs2[buf] + t_lds[n]) = b_reg[n];
+    }
+  };
+  // this wave: rows wm * 64 + {0, 32}; matrix-row blocks fb[0], fb[1] of the tile
+  const int fb[2] = {GATED ? wn * 32 : wn * 64, GATED ? 64 + wn * 32 : wn * 64 + 32};
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  load(0);
+  stash(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += KT) {
+    const bool more = k0 + KT < K;
+    if (more) load(k0 + KT);
+    const T* As = As2[buf];
+    const T* Bs = Bs2[buf];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int kk = s * 2 * MW::kElems + (lane / 32) * MW::kElems;
+      typename MW::Frag xf[2], wf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        xf[i] = *reinterpret_cast<const typename MW::Frag*>(As + (wm * 64 + i * 32 + lane % 32) * LD + kk);
+        wf[i] = *reinterpret_cast<const typename MW::Frag*>(Bs + (fb[i] + lane % 32) * LD + kk);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = MW::mma(wf[j], xf[i], acc[i][j]);
+    }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  // register v of lane l: matrix row 8 * (v / 4) + 4 * (l / 32) + v % 4 of the block, token l % 32
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int place = row0 + wm * 64 + i * 32 + lane % 32;
+    if (place >= row_end) continue;
+    T* orow = out + static_cast<size_t>(place) * ldo;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int f = 8 * (v / 4) + 4 * (lane / 32) + v % 4;
+      if constexpr (GATED) {
+        const int col = c0 + wn * 32 + f;
+        if (col >= N) continue;
+        const float g = fminf(acc[i][0][v], limit);
+        const float u = fminf(fmaxf(acc[i][1][v], -limit), limit);
+        orow[col] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+      } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int col = c0 + wn * 64 + j * 32 + f;
+          if (col < N) orow[col] = from_f32<T>(acc[i][j][v]);
+        }
+      }
     }
   }
 }
@@ -455,43 +663,57 @@ int lyp_moe_route(const float* z, const float* bias, int rows, int E, int top, i
               kMostTop);
   if (rows == 0) return 0;
   LYP_REQUIRE(top < kMostTop || always < 0, "moe_route: %d chosen and one more", top);
-  moe_route_kernel<<<(rows + 3) / 4, 256, 0, stream>>>(z, bias, rows, E, top, idx, wgt, always);
+  moe_route_kernel<<<(rows + 3) / 4, 256, 0, stream>>>(z, bias, rows, E, top, idx, wgt, always, 1);
   LYP_LAUNCH_CHECK("moe_route");
   return 0;
 }
 
 // x [rows, K] in the activations' type, w [E, K] float: the router's logits, the choice and the weights.
+// How many workgroups had better share a row block's inner dimension (1: none; more need `part`,
+// that many * rows * E floats).
+int lyp_moe_route_splits(int rows, int K) {
+  const int blocks = (rows + 15) / 16, steps = (K + 15) / 16;
+  int ks = compute_units() / std::max(blocks, 1);
+  ks = std::min(ks, std::min(16, steps / kRouteWaves));
+  return std::max(ks, 1);
+}
+
 int lyp_moe_route_fused(const void* x, int ldx, int dtype, const float* w, const float* bias, int rows, int E, int K,
-                        int top, int32_t* idx, float* wgt, int always, hipStream_t stream) {
+                        int top, int32_t* idx, float* wgt, int always, float* part, int splits, hipStream_t stream) {
+  LYP_REQUIRE(splits >= 1 && (splits == 1 || part != nullptr), "moe_route: %d shares of the inner dimension", splits);
   LYP_REQUIRE(rows >= 0 && E > 0 && E <= kMostExperts && top > 0 && top <= E && top <= kMostTop && K > 0 && ldx >= K,
               "moe_route: %d rows, %d experts (at most %d), %d chosen (at most %d), inner size %d", rows, E,
               kMostExperts, top, kMostTop, K);
   LYP_REQUIRE(top < kMostTop || always < 0, "moe_route: %d chosen and one more", top);
   if (rows == 0) return 0;
-  const size_t lds = sizeof(float) * (4 * kRouteBlocks * kWave * 4 + 16 * E);
-  const int blocks = (rows + 15) / 16;
+  const size_t lds = sizeof(float) * (kRouteWaves * kRouteBlocks * kWave * 4 + 16 * E);
+  const dim3 blocks((rows + 15) / 16, splits);
+  const int esz = dtype == kF32 ? 4 : 2;
+  const int vec_ok = K % 4 == 0 && ldx % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * esz) == 0 &&
+                     reinterpret_cast<uintptr_t>(w) % 16 == 0;
   if (dtype == kF32)
-    moe_route_fused_kernel<float><<<blocks, 256, lds, stream>>>(static_cast<const float*>(x), ldx, w, bias, rows, E, K,
-                                                                top, idx, wgt, always);
+    moe_route_fused_kernel<float><<<blocks, kRouteWaves * kWave, lds, stream>>>(
+        static_cast<const float*>(x), ldx, w, bias, rows, E, K, top, idx, wgt, always, vec_ok, part);
   else if (dtype == kBF16)
-    moe_route_fused_kernel<bf16_t><<<blocks, 256, lds, stream>>>(static_cast<const bf16_t*>(x), ldx, w, bias, rows, E,
-                                                                 K, top, idx, wgt, always);
+    moe_route_fused_kernel<bf16_t><<<blocks, kRouteWaves * kWave, lds, stream>>>(
+        static_cast<const bf16_t*>(x), ldx, w, bias, rows, E, K, top, idx, wgt, always, vec_ok, part);
   else
     LYP_REQUIRE(false, "moe_route: unknown dtype %d", dtype);
+  if (splits > 1) moe_route_kernel<<<(rows + 3) / 4, 256, 0, stream>>>(part, bias, rows, E, top, idx, wgt, always, splits);
   LYP_LAUNCH_CHECK("moe_route");
   return 0;
 }
 
 // Rows per tile the products had better use for `pairs` pairs over E experts, and the most tiles
 // there can then be (the products' grid).
-int lyp_moe_tile_rows(int pairs, int E) { return pairs >= 32 * E ? 64 : 16; }
+int lyp_moe_tile_rows(int pairs, int E) { return pairs >= 96 * E ? 128 : (pairs >= 32 * E ? 64 : 16); }
 int lyp_moe_most_tiles(int pairs, int E, int tile_rows) {
   return (pairs + tile_rows - 1) / tile_rows + std::min(E, pairs);
 }
 
 int lyp_moe_sort(const int32_t* idx, int pairs, int E, int tile_rows, int32_t* expert_off, int32_t* sorted_pair,
                  int32_t* place_of, int32_t* tile_expert, int32_t* tile_row0, int32_t* n_tiles, hipStream_t stream) {
-  LYP_REQUIRE(pairs >= 0 && E > 0 && E <= kMostExperts && (tile_rows == 16 || tile_rows == 64),
+  LYP_REQUIRE(pairs >= 0 && E > 0 && E <= kMostExperts && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128),
               "moe_sort: %d pairs, %d experts, tiles of %d rows", pairs, E, tile_rows);
   const size_t lds = sizeof(int32_t) * (3 * E + 1 + kSortWaves * E);
   moe_sort_kernel<<<1, kSortThreads, lds, stream>>>(idx, pairs, E, tile_rows, expert_off, sorted_pair, place_of,
@@ -508,9 +730,9 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
                  int K, float limit, float alpha, hipStream_t stream) {
   LYP_REQUIRE(N > 0 && K > 0 && lda >= K && ldw >= K && ldo >= N && top > 0 && most_tiles >= 0,
               "moe_gemm: bad sizes N=%d K=%d lda=%d ldw=%d ldo=%d", N, K, lda, ldw, ldo);
-  LYP_REQUIRE(tile_rows == 16 || tile_rows == 64, "moe_gemm: tiles of %d rows", tile_rows);
+  LYP_REQUIRE(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "moe_gemm: tiles of %d rows", tile_rows);
   if (most_tiles == 0) return 0;
-  const int col_tiles = (N + 63) / 64;
+  const int col_tiles = tile_rows == 128 && !gated ? (N + 127) / 128 : (N + 63) / 64;
   LYP_REQUIRE(col_tiles <= 65535, "moe_gemm: too many columns for one launch");
   const int esz = dtype == kF32 ? 4 : 2;
   const int vec = 16 / esz;
@@ -521,9 +743,16 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
   moe_gemm_kernel<T, MB, G, T><<<grid, 256, 0, stream>>>(                                                       \
       static_cast<const T*>(a), lda, static_cast<const T*>(w), w_expert_stride, ldw, static_cast<T*>(out), ldo, \
       tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok)
+#define LYP_MOE_WIDE(T, G)                                                                                      \
+  moe_gemm_wide_kernel<T, G><<<grid, 256, 0, stream>>>(                                                         \
+      static_cast<const T*>(a), lda, static_cast<const T*>(w), w_expert_stride, ldw, static_cast<T*>(out), ldo, \
+      tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok)
 #define LYP_MOE_T(T)                                 \
   do {                                               \
-    if (tile_rows == 64) {                           \
+    if (tile_rows == 128) {                          \
+      if (gated) LYP_MOE_WIDE(T, true);              \
+      else LYP_MOE_WIDE(T, false);                   \
+    } else if (tile_rows == 64) {                    \
       if (gated) LYP_MOE(T, 4, true);                \
       else LYP_MOE(T, 4, false);                     \
     } else {                                         \
@@ -535,6 +764,7 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
   else if (dtype == kBF16) LYP_MOE_T(bf16_t);
   else LYP_REQUIRE(false, "moe_gemm: unknown dtype %d", dtype);
 #undef LYP_MOE_T
+#undef LYP_MOE_WIDE
 #undef LYP_MOE
   LYP_LAUNCH_CHECK("moe_gemm");
   return 0;

@@ -114,8 +114,9 @@ def core() -> ctypes.CDLL:
                                       c_int, c_int, c_int, c_int, c_void_p]
         lib.lyp_stream_add.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_longlong, c_void_p]
         lib.lyp_moe_route.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]
+        lib.lyp_moe_route_splits.argtypes = [c_int, c_int]
         lib.lyp_moe_route_fused.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                                            c_void_p, c_void_p, c_int, c_void_p]
+                                            c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]
         lib.lyp_moe_tile_rows.argtypes = [c_int, c_int]
         lib.lyp_moe_most_tiles.argtypes = [c_int, c_int, c_int]
         lib.lyp_moe_sort.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -1375,8 +1376,11 @@ def moe_route_from(x: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | N
     idx = torch.empty((T, per), dtype=torch.int32, device=x.device)
     wgt = torch.empty((T, per), dtype=torch.float32, device=x.device)
     lib = core()
+    # few rows: several workgroups share the inner dimension and leave partial sums
+    splits = lib.lyp_moe_route_splits(T, K)
+    part = torch.empty((splits, T, E), dtype=torch.float32, device=x.device) if splits > 1 else None
     _check(lib.lyp_moe_route_fused(_p(x), x.stride(0), _code(x.dtype), _p(router), _p(bias), T, E, K, top, _p(idx),
-                                   _p(wgt), int(always), _stream()), lib)
+                                   _p(wgt), int(always), _p(part), splits, _stream()), lib)
     return idx, wgt
 
 
