@@ -260,12 +260,26 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
       tile_row0[tbase[e] + i] = base[e] + i * tile_rows;
     }
   }
+  // a thread's experts of the next rounds are asked for ahead, kAhead rounds at a time
+  constexpr int kAhead = 8;
+  int mine[kAhead];
   for (int p0 = 0; p0 < P; p0 += kSortThreads) {
+    const int round = p0 / kSortThreads;
+    if (round % kAhead == 0) {
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) {
+        const int pa = p0 + a * kSortThreads + tid;
+        mine[a] = pa < P ? idx[pa] : -1;
+      }
+    }
     __syncthreads();
     for (int i = tid; i < kSortWaves * E; i += kSortThreads) wcnt[i] = 0;
     __syncthreads();
     const int p = p0 + tid;
-    const int e = p < P ? idx[p] : -1;
+    int e = -1;
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+      if (round % kAhead == a) e = mine[a];
     int rank = 0;
     bool last = true;
     for (int l = 0; l < kWave; ++l) {
@@ -606,44 +620,61 @@ __global__ void glu_clamped_kernel(const T* __restrict__ gate_up, T* __restrict_
 }
 
 // out [rows, H] float = addend + shared + sum_k wgt[row, k] * y[place_of[row * top + k]]
-// One workgroup a row; the row's places and weights are read once, and every thread then has
-// several columns' loads in flight at a time.
-template <typename T>
+// One workgroup a row; the row's places and weights are read once; a thread takes V neighbouring
+// columns at a time (V = 4 where rows are whole multiples of that, else 1), two such groups in flight.
+template <typename T, int V>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int32_t* __restrict__ place_of,
                                    const float* __restrict__ wgt, int top, const T* __restrict__ addend,
                                    const T* __restrict__ shared, float* __restrict__ out, int rows, int H) {
   __shared__ int32_t s_at[kMostTop];
   __shared__ float s_w[kMostTop];
+  typedef T VecT __attribute__((ext_vector_type(V)));
+  typedef float VecF __attribute__((ext_vector_type(V)));
   const int row = blockIdx.x;
   if (threadIdx.x < top) {
     s_at[threadIdx.x] = place_of[static_cast<size_t>(row) * top + threadIdx.x];
     s_w[threadIdx.x] = wgt[static_cast<size_t>(row) * top + threadIdx.x];
   }
   __syncthreads();
-  constexpr int U = 4;
-  for (int c0 = threadIdx.x; c0 < H; c0 += U * blockDim.x) {
-    float v[U];
+  constexpr int U = 2;
+  const int stride = blockDim.x * V;
+  auto get = [&](const T* p) {
+    VecF f;
+    if constexpr (V == 1) {
+      f[0] = to_f32(p[0]);
+    } else {
+      const VecT v = *reinterpret_cast<const VecT*>(p);
+#pragma unroll
+      for (int i = 0; i < V; ++i) f[i] = to_f32(v[i]);
+    }
+    return f;
+  };
+  for (int c0 = threadIdx.x * V; c0 < H; c0 += U * stride) {
+    VecF v[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int c = c0 + u * blockDim.x;
-      v[u] = 0.f;
+      const int c = c0 + u * stride;
+#pragma unroll
+      for (int i = 0; i < V; ++i) v[u][i] = 0.f;
       if (c >= H) continue;
-      if (addend != nullptr) v[u] += to_f32(addend[static_cast<size_t>(row) * H + c]);
-      if (shared != nullptr) v[u] += to_f32(shared[static_cast<size_t>(row) * H + c]);
+      if (addend != nullptr) v[u] += get(addend + static_cast<size_t>(row) * H + c);
+      if (shared != nullptr) v[u] += get(shared + static_cast<size_t>(row) * H + c);
     }
     for (int k = 0; k < top; ++k) {
       const size_t base = static_cast<size_t>(s_at[k]) * H;
       const float wk = s_w[k];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int c = c0 + u * blockDim.x;
-        if (c < H) v[u] += wk * to_f32(y[base + c]);
+        const int c = c0 + u * stride;
+        if (c < H) v[u] += wk * get(y + base + c);
       }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int c = c0 + u * blockDim.x;
-      if (c < H) out[static_cast<size_t>(row) * H + c] = v[u];
+      const int c = c0 + u * stride;
+      if (c >= H) continue;
+      if constexpr (V == 1) out[static_cast<size_t>(row) * H + c] = v[u][0];
+      else *reinterpret_cast<VecF*>(out + static_cast<size_t>(row) * H + c) = v[u];
     }
   }
 }
@@ -793,17 +824,24 @@ int lyp_moe_combine(const void* y, const int32_t* place_of, const float* wgt, in
   LYP_REQUIRE(rows >= 0 && H > 0 && top > 0, "moe_combine: bad sizes");
   if (rows == 0) return 0;
   LYP_REQUIRE(top <= kMostTop, "moe_combine: %d choices a token (at most %d)", top, kMostTop);
-  const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 128);
-  if (dtype == kF32)
-    moe_combine_kernel<float><<<rows, threads, 0, stream>>>(static_cast<const float*>(y), place_of, wgt, top,
-                                                            static_cast<const float*>(addend),
-                                                            static_cast<const float*>(shared), out, rows, H);
-  else if (dtype == kBF16)
-    moe_combine_kernel<bf16_t><<<rows, threads, 0, stream>>>(static_cast<const bf16_t*>(y), place_of, wgt, top,
-                                                             static_cast<const bf16_t*>(addend),
-                                                             static_cast<const bf16_t*>(shared), out, rows, H);
-  else
+  const bool vec = H % 4 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 && reinterpret_cast<uintptr_t>(addend) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(shared) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const int per = vec ? 4 : 1;
+  const int threads = H / per >= 512 ? 256 : (H / per >= 128 ? 128 : 64);
+#define LYP_COMBINE(T, V)                                                                                      \
+  moe_combine_kernel<T, V><<<rows, threads, 0, stream>>>(static_cast<const T*>(y), place_of, wgt, top,        \
+                                                        static_cast<const T*>(addend),                       \
+                                                        static_cast<const T*>(shared), out, rows, H)
+  if (dtype == kF32) {
+    if (vec) LYP_COMBINE(float, 4);
+    else LYP_COMBINE(float, 1);
+  } else if (dtype == kBF16) {
+    if (vec) LYP_COMBINE(bf16_t, 4);
+    else LYP_COMBINE(bf16_t, 1);
+  } else {
     LYP_REQUIRE(false, "moe_combine: unknown dtype %d", dtype);
+  }
+#undef LYP_COMBINE
   LYP_LAUNCH_CHECK("moe_combine");
   return 0;
 }

@@ -41,27 +41,37 @@ __global__ void qk_norm_rope_kv_kernel(T* __restrict__ qkv, int ld, const float*
                                        const int32_t* __restrict__ positions, const float* __restrict__ table,
                                        int rot, const int32_t* __restrict__ slot_map, T* __restrict__ kpool,
                                        T* __restrict__ vpool, int H, int G, int D, int V, int bs) {
-  __shared__ float scratch[16];
   const int t = blockIdx.x;
   T* row = qkv + static_cast<size_t>(t) * ld;
   const int nq = H * D, nk = G * D;
-  float inv_q = 1.f, inv_k = 1.f;
-  if (wq != nullptr) {
-    float s = 0.f;
+  // both sums of squares in one pass and one reduction (wave by wave, in the waves' order)
+  __shared__ float s_sum[2][16];
+  float sq = 0.f, sk = 0.f;
+  if (wq != nullptr)
     for (int i = threadIdx.x; i < nq; i += blockDim.x) {
       const float v = to_f32(row[i]);
-      s += v * v;
+      sq += v * v;
     }
-    inv_q = 1.0f / sqrtf(block_sum(s, scratch) / static_cast<float>(nq) + eps);
-  }
-  if (wk != nullptr) {
-    float s = 0.f;
+  if (wk != nullptr)
     for (int i = threadIdx.x; i < nk; i += blockDim.x) {
       const float v = to_f32(row[nq + i]);
-      s += v * v;
+      sk += v * v;
     }
-    inv_k = 1.0f / sqrtf(block_sum(s, scratch) / static_cast<float>(nk) + eps);
+  sq = wave_sum(sq);
+  sk = wave_sum(sk);
+  if (threadIdx.x % kWave == 0) {
+    s_sum[0][threadIdx.x / kWave] = sq;
+    s_sum[1][threadIdx.x / kWave] = sk;
   }
+  __syncthreads();
+  sq = sk = 0.f;
+  for (int wv = 0; wv < static_cast<int>(blockDim.x) / kWave; ++wv) {
+    sq += s_sum[0][wv];
+    sk += s_sum[1][wv];
+  }
+  const float inv_q = wq != nullptr ? 1.0f / sqrtf(sq / static_cast<float>(nq) + eps) : 1.f;
+  const float inv_k = wk != nullptr ? 1.0f / sqrtf(sk / static_cast<float>(nk) + eps) : 1.f;
+  __syncthreads();   // every thread has read the row's values it summed before anyone writes queries back
   const float* cs = rot > 0 ? table + static_cast<size_t>(positions[t]) * rot : nullptr;
   const int half = rot / 2;
   const int per = D / 2 + (D & 1);   // pairs of a head (the last one single when D is odd)
@@ -96,6 +106,86 @@ __global__ void qk_norm_rope_kv_kernel(T* __restrict__ qkv, int ld, const float*
     dst[0] = from_f32<T>(a);
     if (two) dst[1] = from_f32<T>(b);
   }
+  const T* vrow = row + nq + nk;
+  for (int idx = threadIdx.x; idx < G * V; idx += blockDim.x) {
+    const int g = idx / V, d = idx % V;
+    vpool[((static_cast<size_t>(page) * G + g) * V + d) * bs + off] = vrow[idx];
+  }
+}
+
+// The same with 16 bytes a thread and access: head sizes, the rotated width and the row's stride are
+// whole multiples of the 16 bytes' values, so a thread's values are whole pairs of one head and
+// either all rotate or none.
+template <typename T>
+__global__ void qk_norm_rope_kv_vec_kernel(T* __restrict__ qkv, int ld, const float* __restrict__ wq,
+                                           const float* __restrict__ wk, float eps,
+                                           const int32_t* __restrict__ positions, const float* __restrict__ table,
+                                           int rot, const int32_t* __restrict__ slot_map, T* __restrict__ kpool,
+                                           T* __restrict__ vpool, int H, int G, int D, int V, int bs) {
+  constexpr int VEC = 16 / sizeof(T);
+  typedef T VecT __attribute__((ext_vector_type(VEC)));
+  const int t = blockIdx.x;
+  T* row = qkv + static_cast<size_t>(t) * ld;
+  const int nq = H * D, nk = G * D;
+  __shared__ float s_sum[2][16];
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x * VEC; i < nq + nk; i += blockDim.x * VEC) {
+    const VecT x = *reinterpret_cast<const VecT*>(row + i);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) ss += to_f32(x[e]) * to_f32(x[e]);
+    if (i < nq) sq += ss;
+    else sk += ss;
+  }
+  sq = wave_sum(sq);
+  sk = wave_sum(sk);
+  if (threadIdx.x % kWave == 0) {
+    s_sum[0][threadIdx.x / kWave] = sq;
+    s_sum[1][threadIdx.x / kWave] = sk;
+  }
+  __syncthreads();
+  sq = sk = 0.f;
+  for (int wv = 0; wv < static_cast<int>(blockDim.x) / kWave; ++wv) {
+    sq += s_sum[0][wv];
+    sk += s_sum[1][wv];
+  }
+  const float inv_q = wq != nullptr ? 1.0f / sqrtf(sq / static_cast<float>(nq) + eps) : 1.f;
+  const float inv_k = wk != nullptr ? 1.0f / sqrtf(sk / static_cast<float>(nk) + eps) : 1.f;
+  __syncthreads();
+  const float* cs = rot > 0 ? table + static_cast<size_t>(positions[t]) * rot : nullptr;
+  const int half = rot / 2;
+  const int slot = slot_map != nullptr ? slot_map[t] : -1;
+  const int page = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
+  for (int i = threadIdx.x * VEC; i < nq + nk; i += blockDim.x * VEC) {
+    const bool is_q = i < nq;
+    if (!is_q && slot < 0) continue;
+    const int e0 = is_q ? i : i - nq;            // place within the projection
+    const int d0 = e0 % D;                       // place within the head
+    const float* wn = is_q ? wq : wk;
+    const float inv = is_q ? inv_q : inv_k;
+    const VecT x = *reinterpret_cast<const VecT*>(row + i);
+    float v[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) v[e] = to_f32(x[e]) * inv;
+    if (wn != nullptr) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[e] *= wn[e0 + e];
+    }
+    if (d0 < rot) {
+#pragma unroll
+      for (int e = 0; e < VEC; e += 2) {
+        const int pi = (d0 + e) / 2;
+        rotate_pair(v[e], v[e + 1], cs[pi], cs[half + pi], v[e], v[e + 1]);
+      }
+    }
+    VecT y;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) y[e] = from_f32<T>(v[e]);
+    if (is_q) *reinterpret_cast<VecT*>(row + i) = y;
+    else
+      *reinterpret_cast<VecT*>(kpool + ((static_cast<size_t>(page) * G + e0 / D) * bs + off) * D + d0) = y;
+  }
+  if (slot < 0) return;
   const T* vrow = row + nq + nk;
   for (int idx = threadIdx.x; idx < G * V; idx += blockDim.x) {
     const int g = idx / V, d = idx % V;
@@ -216,14 +306,22 @@ int lyp_qk_norm_rope_kv(void* qkv, int ld, int dtype, const float* wq, const flo
               "qk_norm_rope_kv: %d rotated values of %d", rot, D);
   LYP_REQUIRE(slot_map == nullptr || (kpool != nullptr && vpool != nullptr && bs > 0), "qk_norm_rope_kv: no pools");
   if (n_rows == 0) return 0;
-  const int threads = H * D >= 2048 ? 512 : 256;
-#define LYP_QKN(T)                                                                                              \
-  qk_norm_rope_kv_kernel<T><<<n_rows, threads, 0, stream>>>(static_cast<T*>(qkv), ld, wq, wk, eps, positions,   \
-                                                           table, rot, slot_map, static_cast<T*>(kpool),       \
-                                                           static_cast<T*>(vpool), H, G, D, V, bs)
-  if (dtype == kF32) LYP_QKN(float);
-  else if (dtype == kBF16) LYP_QKN(bf16_t);
-  else LYP_REQUIRE(false, "qk_norm_rope_kv: unknown dtype %d", dtype);
+  LYP_REQUIRE(dtype == kF32 || dtype == kBF16, "qk_norm_rope_kv: unknown dtype %d", dtype);
+  const int vec = dtype == kF32 ? 4 : 8;
+  const bool wide = D % vec == 0 && rot % vec == 0 && ld % vec == 0 && reinterpret_cast<uintptr_t>(qkv) % 16 == 0 &&
+                    (kpool == nullptr || reinterpret_cast<uintptr_t>(kpool) % 16 == 0);
+  const int work = wide ? (H + G) * D / vec : H * D / 2;
+  const int threads = work >= 512 ? 512 : (work >= 256 ? 256 : 128);
+#define LYP_QKN(KERNEL, T)                                                                                \
+  KERNEL<T><<<n_rows, threads, 0, stream>>>(static_cast<T*>(qkv), ld, wq, wk, eps, positions, table, rot, \
+                                            slot_map, static_cast<T*>(kpool), static_cast<T*>(vpool), H, G, D, V, bs)
+  if (dtype == kF32) {
+    if (wide) LYP_QKN(qk_norm_rope_kv_vec_kernel, float);
+    else LYP_QKN(qk_norm_rope_kv_kernel, float);
+  } else {
+    if (wide) LYP_QKN(qk_norm_rope_kv_vec_kernel, bf16_t);
+    else LYP_QKN(qk_norm_rope_kv_kernel, bf16_t);
+  }
 #undef LYP_QKN
   LYP_LAUNCH_CHECK("qk_norm_rope_kv");
   return 0;

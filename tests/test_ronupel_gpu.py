@@ -215,7 +215,8 @@ def test_the_given_shape_of_things_is_not_assumed(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("layers", ["many experts", "no feed-forward at all", "looped four times from the start", "heads of 128"])
+@pytest.mark.parametrize("layers", ["many experts", "no feed-forward at all", "looped four times from the start", "heads of 128",
+                                    "rows of no whole 16 bytes", "heads of 80 and of 256"])
 def test_other_orders_and_sizes(tmp_path, dtype, layers):
     if layers == "many experts":
         cfg = config(111, 64, [attn(2, 1, 16, 16, window=17, keep=2, dims=8, scale=0.5, mlp=moe(70, 5, 8, 3.0, shared=(24, 3.0)))])
@@ -225,6 +226,12 @@ def test_other_orders_and_sizes(tmp_path, dtype, layers):
         cfg = config(111, 64, [attn(4, 4, 16, 16, window=8, keep=8, dims=16, factor=8.0, scale=0.5, mlp=moe(4, 2, 24, 2.0)),
                                attn(2, 1, 32, 32, window=30, keep=0, dims=2, scale=0.3, mlp=moe(2, 1, 16, 2.0, shared=(8, 2.0)))],
                      loop=(0, 2, 4))
+    elif layers == "rows of no whole 16 bytes":
+        cfg = config(111, 100, [attn(5, 5, 12, 20, window=11, keep=3, dims=6, factor=2.0, scale=0.5, mlp=moe(3, 2, 36, 2.0, shared=(52, 1.0))),
+                                attn(2, 1, 18, 18, window=25, keep=2, dims=18, scale=0.4, mlp=moe(5, 1, 44, 3.0))])
+    elif layers == "heads of 80 and of 256":
+        cfg = config(111, 64, [attn(2, 2, 80, 80, window=19, keep=2, dims=40, factor=4.0, scale=0.2, mlp=moe(3, 1, 32, 2.0)),
+                               attn(1, 1, 256, 256, window=70, keep=1, dims=128, scale=0.1)])
     else:
         cfg = config(111, 128, [attn(2, 1, 128, 128, window=50, keep=4, dims=64, factor=2.0, scale=0.2, mlp=moe(4, 2, 64, 2.0))])
     folder = write_model(str(tmp_path / "m"), cfg, seed=9, dtype=dtype)
@@ -235,7 +242,7 @@ def test_other_orders_and_sizes(tmp_path, dtype, layers):
     for _ in range(2):
         t.step([("x", 1), ("y", 1)])
     t.step([("x", 45)], end=["x", "y"])
-    check_folder(t, run_folder(folder, dtype, t, block_size=8 if layers != "heads of 128" else 16), folder, dtype, layers)
+    check_folder(t, run_folder(folder, dtype, t, block_size=8 if "heads of" not in layers else 16), folder, dtype, layers)
 
 
 # ------------------------------------------------------------------- generation
