@@ -51,7 +51,7 @@ CONFIGS = {
                           attn(2, 2, 6, 30, window=3, keep=7, dims=2, base=50.0, factor=1.5, scale=0.8,
                                mlp=moe(3, 3, 20, 0.7))],
                 loop=(0, 2, 2), eps=1e-5),
-    "B": config(150, 128, [attn(4, 2, 32, 32, window=21, keep=3, dims=16, base=20000.0, factor=4.0, scale=0.35,
+    "B": config(150, 128, [attn(4, 2, 32, 32, window=21, keep=3, dims=16, base=30000.0, factor=4.0, scale=0.35,
                                 mlp=moe(8, 8, 48, 2.5)),
                            attn(2, 2, 16, 16, window=100, keep=70, dims=16, base=300.0, scale=0.5,
                                 mlp=moe(6, 1, 80, 4.0, shared=(64, 1.0)))],

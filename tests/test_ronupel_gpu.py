@@ -221,7 +221,7 @@ def test_other_orders_and_sizes(tmp_path, dtype, layers):
     if layers == "many experts":
         cfg = config(111, 64, [attn(2, 1, 16, 16, window=17, keep=2, dims=8, scale=0.5, mlp=moe(70, 5, 8, 3.0, shared=(24, 3.0)))])
     elif layers == "no feed-forward at all":
-        cfg = config(111, 48, [attn(2, 2, 12, 12, window=6, keep=1, scale=0.6), attn(3, 1, 16, 16, window=40, keep=4, scale=0.5)])
+        cfg = config(111, 48, [attn(2, 2, 12, 12, window=6, keep=1, scale=0.6), attn(3, 1, 16, 16, window=44, keep=5, scale=0.5)])
     elif layers == "looped four times from the start":
         cfg = config(111, 64, [attn(4, 4, 16, 16, window=8, keep=8, dims=16, factor=8.0, scale=0.5, mlp=moe(4, 2, 24, 2.0)),
                                attn(2, 1, 32, 32, window=30, keep=0, dims=2, scale=0.3, mlp=moe(2, 1, 16, 2.0, shared=(8, 2.0)))],

@@ -79,11 +79,11 @@ def test_position_table_with_divided_frequencies():
     """The 64-bit table is the nearest float to cos and sin of position * base^(-2i/d) / factor, far out too."""
     from lyapunov_engine_amd.parts.rope import RotaryEncoding
 
-    enc = RotaryEncoding(6, 20000.0, 5000, scaling={"rope_type": "linear", "factor": 8.0}, precise=True)
+    enc = RotaryEncoding(6, 30000.0, 5000, scaling={"rope_type": "linear", "factor": 6.0}, precise=True)
     enc.materialize(DEV, torch.float32)
     for p in (0, 1, 63, 4999):
         for i in range(3):
-            a = p * 20000.0 ** (-2.0 * i / 6) / 8.0
+            a = p * 30000.0 ** (-2.0 * i / 6) / 6.0
             assert abs(float(enc.table[p, i]) - math.cos(a)) < 1e-7 and abs(float(enc.table[p, 3 + i]) - math.sin(a)) < 1e-7
 
 
@@ -189,7 +189,7 @@ CASES = [  # kernel, heads, kv heads, key size, value size, page
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("case", CASES)
-@pytest.mark.parametrize("mask", [(0, 0), (40, 4), (5, 0), (17, 70), (64, 16), (1, 1), (200, 3)])
+@pytest.mark.parametrize("mask", [(0, 0), (44, 5), (5, 0), (17, 70), (64, 16), (1, 1), (200, 3)])
 def test_attention_over_pages(dtype, case, mask):
     """Random keys: whole prompts, a portion at the end of a long context, and the pages behind the
     window already given back."""
@@ -206,7 +206,7 @@ def test_attention_over_pages(dtype, case, mask):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("sizes", [(4, 2, 32, 16), (2, 1, 64, 16), (3, 3, 16, 4), (16, 1, 16, 16), (2, 2, 128, 16)])
-@pytest.mark.parametrize("mask", [(0, 0), (40, 4), (300, 0), (17, 70), (64, 300), (1, 0)])
+@pytest.mark.parametrize("mask", [(0, 0), (44, 5), (300, 0), (17, 70), (64, 300), (1, 0)])
 @pytest.mark.parametrize("n", [1, 5, 256, 257, 700, 1100])
 def test_one_new_token_over_partitions(dtype, sizes, mask, n):
     H, G, D, page = sizes
@@ -221,7 +221,7 @@ def test_one_new_token_over_partitions(dtype, sizes, mask, n):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("kernel", ["rows", "tiles", "split"])
-@pytest.mark.parametrize("mask", [(40, 4), (64, 1), (9, 17), (130, 66)])
+@pytest.mark.parametrize("mask", [(44, 5), (64, 1), (9, 17), (130, 66)])
 def test_a_planted_key_is_found_exactly_where_the_mask_allows(dtype, kernel, mask):
     """One key that the last query matches far better than any other, planted in turn at every
     place of interest: the window's two edges, the kept tokens' edge, page and tile edges, the
