@@ -593,7 +593,7 @@ struct WideTile {
 // with a row of ones), and return the probabilities as the column operand of the P.V product.
 template <bool MASKED, int NB>
 __device__ __forceinline__ void softmax_wide(const f32x4 (&s)[NB], bf16x8 (&pw)[NB / 2], float scale_log2, int kb0,
-                                             int pos, int window, int hi, float& m_run, f32x4& lacc,
+                                             int pos, int window, int keep, int hi, float& m_run, f32x4& lacc,
                                              f32x4 (&o)[kSteps], int lane) {
   bool vis[NB][4];
   float mx = LYP_NEG_INF;
@@ -603,7 +603,7 @@ __device__ __forceinline__ void softmax_wide(const f32x4 (&s)[NB], bf16x8 (&pw)[
     for (int i = 0; i < 4; ++i) {
       if constexpr (MASKED) {
         const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
-        vis[u][i] = key <= pos && key < hi && (window == 0 || key > pos - window);
+        vis[u][i] = key <= pos && key < hi && (window == 0 || key > pos - window || key < keep);
         mx = fmaxf(mx, vis[u][i] ? s[u][i] : LYP_NEG_INF);
       } else {
         vis[u][i] = true;
@@ -656,7 +656,7 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int n_tiles, int nh, int nkv,
     int bs, int window, float scale_log2, const float* __restrict__ sink, int paired, float* __restrict__ part_o,
     float* __restrict__ part_ml,
-    int n_parts) {
+    int n_parts, int keep) {
   using T = bf16_t;
   using WT = WideTile;
   using MMA = Mma16Wide<bf16_t>;
@@ -817,11 +817,11 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
         bf16x8 kx = r.k[n], vx = r.v[n];
         if (!inside || r.lost[n]) {
           const int key = kt0 + p_key[n];
-          if (key < lo_wg || key >= hi_wg || r.lost[n]) kx = zero_vec();
+          if ((key < lo_wg && key >= keep) || key >= hi_wg || r.lost[n]) kx = zero_vec();
           const int key0 = kt0 + p_vkey[n];
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (key0 + e < lo_wg || key0 + e >= hi_wg || r.lost[n]) vx[e] = from_f32<T>(0.f);
+            if ((key0 + e < lo_wg && key0 + e >= keep) || key0 + e >= hi_wg || r.lost[n]) vx[e] = from_f32<T>(0.f);
         }
         if (!p_live[n]) continue;
         *reinterpret_cast<bf16x8*>(ks + k_lds[n]) = kx;
@@ -853,10 +853,10 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
       const bool full = kt0 + KT - 1 <= pos0 && kt0 >= lo_wg && pos0 + 15 <= pos_last_wg &&
                         (window == 0 || kt0 > pos0 + 15 - window);
       if (full)
-        softmax_wide<false, NB>(sc, pw, scale_log2, kt0, pos0 + col, window, hi_wg, m_run, lacc, o, lane);
+        softmax_wide<false, NB>(sc, pw, scale_log2, kt0, pos0 + col, window, keep, hi_wg, m_run, lacc, o, lane);
       else
-        softmax_wide<true, NB>(sc, pw, scale_log2, kt0, col_valid ? pos0 + col : -1, window, hi_wg, m_run, lacc, o,
-                               lane);
+        softmax_wide<true, NB>(sc, pw, scale_log2, kt0, col_valid ? pos0 + col : -1, window, keep, hi_wg, m_run, lacc,
+                               o, lane);
 #pragma unroll
       for (int w = 0; w < NWIDE; ++w) {
         lacc = MMA::mma(ones, pw[w], lacc);
@@ -884,6 +884,29 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
       if (kt0 + KSTEP < kt_end) stash(ready, WT::kBufs == 2 ? buf ^ 1 : 0, kt0 + KSTEP);
       __syncthreads();
     };
+
+    // Kept first tokens that the window no longer covers: their tiles come first, one at a time
+    // (few keys: no loads ahead), through set 0's first buffer; the walk below starts at the window.
+    const int kt_window = (lo_wg / KT) * KT;
+    const int kept_end = (n_parts == 1 || blockIdx.z == 0) ? min((keep + KT - 1) / KT * KT, kt_window) : 0;
+    for (int kt0 = 0; kt0 < kept_end; kt0 += KT) {
+      if (set == 0) {
+        TileRegs<PER> rk;
+        int pg[PER], po[PER];
+#pragma unroll
+        for (int n = 0; n < PER; ++n) {
+          const int x = kt0 + 16 * p_blk[n];
+          const int b = x / bs;
+          pg[n] = table[min(b, blk_last)];
+          po[n] = x - b * bs;
+        }
+        ask(rk, pg, po);
+        stash(rk, 0, kt0);
+      }
+      __syncthreads();
+      if (set == 0 && wave_active) compute(0, kt0);
+      __syncthreads();
+    }
 
     TileRegs<PER> ra, rb;
     read_table(page, page_off);
@@ -1391,8 +1414,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   } while (0)
   constexpr int kQB4 = LYP_PREFILL_QB;
 #if LYP_HEAD_DIM % 32 == 0 && !defined(LYP_PREFILL_NARROW)
-  // (the walk of the wide kernel knows no kept first tokens: a window with some takes the kernel above)
-  if (dtype == kBF16 && q_stride % 8 == 0 && bs % 16 == 0 && keep == 0) {
+  if (dtype == kBF16 && q_stride % 8 == 0 && bs % 16 == 0) {
     // Bit 0 of `pair` is the caller's word on whether the tiles differ much in the keys they see
     // (0: no); bit 1 forbids the two sets of waves per unit (for tests and measurements).
     // Units (workgroups before pairing) beyond one per compute unit share compute units anyway;
@@ -1401,7 +1423,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   attn_prefill_wide_kernel<GH, NW, KS><<<grid, NW * KS * kWave, 0, stream>>>(                                 \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), out_stride, kpool, vpool,           \
       block_tables, max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window,            \
-      scale_log2, sink, paired, part_o, part_ml, n_parts)
+      scale_log2, sink, paired, part_o, part_ml, n_parts, keep)
     // Two sets of waves per unit while the launch has at most `kSplitBelow` workgroups per
     // compute unit: its time is then that of the unit with most keys, not of the sum.
 #define LYP_PREFILL_WIDE(GH, NW)                                                                              \
