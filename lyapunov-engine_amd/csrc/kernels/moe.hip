@@ -223,22 +223,61 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void moe_route_fused_kernel(
   }
 }
 
+// The lanes of the wave that hold the same value as this one, as a mask: one ballot per bit of the
+// values (`bits` of them) instead of one look at every lane.
+__device__ __forceinline__ unsigned long long wave_same(int v, int bits) {
+  unsigned long long mask = ~0ull;
+  for (int b = 0; b < bits; ++b) {
+    const unsigned long long set = __builtin_amdgcn_ballot_w64(((v >> b) & 1) != 0);
+    mask &= ((v >> b) & 1) ? set : ~set;
+  }
+  return mask;
+}
+
 constexpr int kSortThreads = 1024;
 constexpr int kSortWaves = kSortThreads / kWave;
 
+// What the sort may do first, for steps of few rows (one kernel less): add up the router's partial
+// sums and choose, as moe_route_kernel does, a wave a row.
+struct RouteFirst {
+  const float* part;     // nullptr: the choices are there already
+  const float* bias;
+  float* wgt;
+  int parts, rows, experts, top, always;
+};
+
 __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
-    const int32_t* __restrict__ idx, int P, int E, int tile_rows, int32_t* __restrict__ expert_off,
+    int32_t* __restrict__ idx, int P, int E, int tile_rows, int32_t* __restrict__ expert_off,
     int32_t* __restrict__ sorted_pair, int32_t* __restrict__ place_of, int32_t* __restrict__ tile_expert,
-    int32_t* __restrict__ tile_row0, int32_t* __restrict__ n_tiles) {
+    int32_t* __restrict__ tile_row0, int32_t* __restrict__ n_tiles, RouteFirst first) {
   extern __shared__ int32_t s_sort[];
   int32_t* cnt = s_sort;               // [E]
   int32_t* base = cnt + E;             // [E]
   int32_t* tbase = base + E;           // [E + 1]
   int32_t* wcnt = tbase + E + 1;       // [kSortWaves][E]
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  int bits = 1;                       // bits that tell the experts (and -1) apart
+  while ((1 << bits) <= E) ++bits;
+  if (first.part != nullptr) {
+    const int per = first.top + (first.always >= 0 ? 1 : 0);
+    for (int row = wave; row < first.rows; row += kSortWaves)
+      route_row(first.part + static_cast<size_t>(row) * first.experts, first.bias, first.experts, first.top,
+                idx + static_cast<size_t>(row) * per, first.wgt + static_cast<size_t>(row) * per, lane, first.always,
+                first.parts, static_cast<size_t>(first.rows) * first.experts);
+    __syncthreads();   // the choices are read back below by other threads of this workgroup
+  }
   for (int e = tid; e < E; e += kSortThreads) cnt[e] = 0;
   __syncthreads();
-  for (int p = tid; p < P; p += kSortThreads) atomicAdd(&cnt[idx[p]], 1);   // integer counts: no order to depend on
+  // counts: a wave first finds out how many of its 64 pairs go to each expert, and one lane per expert
+  // adds that to the expert's count (integers: no order to depend on; 64 lanes adding to a few dozen
+  // places one by one is what this pass would otherwise wait for)
+  for (int p0 = 0; p0 < P; p0 += kSortThreads) {
+    const int p = p0 + tid;
+    const int e = p < P ? idx[p] : -1;                       // (-1: all bits set, a value no expert has)
+    const unsigned long long mates = wave_same(e, bits);
+    const bool last = (mates >> lane) == 1ull;               // no later lane holds the same expert
+    if (e >= 0 && last) atomicAdd(&cnt[e], __builtin_popcountll(mates));
+  }
   __syncthreads();
   if (tid == 0) {
     int run = 0, tiles = 0;
@@ -280,15 +319,9 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
 #pragma unroll
     for (int a = 0; a < kAhead; ++a)
       if (round % kAhead == a) e = mine[a];
-    int rank = 0;
-    bool last = true;
-    for (int l = 0; l < kWave; ++l) {
-      const int el = __shfl(e, l, kWave);
-      if (el == e) {
-        if (l < lane) ++rank;
-        if (l > lane) last = false;
-      }
-    }
+    const unsigned long long mates = wave_same(e, bits);
+    const int rank = __builtin_popcountll(mates & ((1ull << lane) - 1ull));   // earlier lanes with the same expert
+    const bool last = (mates >> lane) == 1ull;
     if (e >= 0 && last) wcnt[wave * E + e] = rank + 1;
     __syncthreads();
     if (e >= 0) {
@@ -753,7 +786,8 @@ int lyp_moe_route_splits(int rows, int K) {
 }
 
 int lyp_moe_route_fused(const void* x, int ldx, int dtype, const float* w, const float* bias, int rows, int E, int K,
-                        int top, int32_t* idx, float* wgt, int always, float* part, int splits, hipStream_t stream) {
+                        int top, int32_t* idx, float* wgt, int always, float* part, int splits, int choose,
+                        hipStream_t stream) {
   LYP_REQUIRE(splits >= 1 && (splits == 1 || part != nullptr), "moe_route: %d shares of the inner dimension", splits);
   LYP_REQUIRE(rows >= 0 && E > 0 && E <= kMostExperts && top > 0 && top <= E && top <= kMostTop && K > 0 && ldx >= K,
               "moe_route: %d rows, %d experts (at most %d), %d chosen (at most %d), inner size %d", rows, E,
@@ -773,7 +807,9 @@ int lyp_moe_route_fused(const void* x, int ldx, int dtype, const float* w, const
         static_cast<const bf16_t*>(x), ldx, w, bias, rows, E, K, top, idx, wgt, always, vec_ok, part);
   else
     LYP_REQUIRE(false, "moe_route: unknown dtype %d", dtype);
-  if (splits > 1) moe_route_kernel<<<(rows + 3) / 4, 256, 0, stream>>>(part, bias, rows, E, top, idx, wgt, always, splits);
+  // (choose == 0 with splits > 1: the caller adds the partial sums up and chooses, lyp_moe_route_sort)
+  if (splits > 1 && choose)
+    moe_route_kernel<<<(rows + 3) / 4, 256, 0, stream>>>(part, bias, rows, E, top, idx, wgt, always, splits);
   LYP_LAUNCH_CHECK("moe_route");
   return 0;
 }
@@ -790,9 +826,30 @@ int lyp_moe_sort(const int32_t* idx, int pairs, int E, int tile_rows, int32_t* e
   LYP_REQUIRE(pairs >= 0 && E > 0 && E <= kMostExperts && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128),
               "moe_sort: %d pairs, %d experts, tiles of %d rows", pairs, E, tile_rows);
   const size_t lds = sizeof(int32_t) * (3 * E + 1 + kSortWaves * E);
-  moe_sort_kernel<<<1, kSortThreads, lds, stream>>>(idx, pairs, E, tile_rows, expert_off, sorted_pair, place_of,
-                                                    tile_expert, tile_row0, n_tiles);
+  moe_sort_kernel<<<1, kSortThreads, lds, stream>>>(const_cast<int32_t*>(idx), pairs, E, tile_rows, expert_off,
+                                                    sorted_pair, place_of, tile_expert, tile_row0, n_tiles,
+                                                    RouteFirst{nullptr, nullptr, nullptr, 0, 0, 0, 0, -1});
   LYP_LAUNCH_CHECK("moe_sort");
+  return 0;
+}
+
+// The same after the choice itself, for few rows: part [parts][rows][experts] are the router's partial
+// sums (lyp_moe_route_fused with choose == 0 left them); idx and wgt [rows][top (+ 1)] are written here.
+int lyp_moe_route_sort(const float* part, int parts, const float* bias, int rows, int experts, int top, int always,
+                       int32_t* idx, float* wgt, int E, int tile_rows, int32_t* expert_off, int32_t* sorted_pair,
+                       int32_t* place_of, int32_t* tile_expert, int32_t* tile_row0, int32_t* n_tiles,
+                       hipStream_t stream) {
+  const int pairs = rows * (top + (always >= 0 ? 1 : 0));
+  LYP_REQUIRE(part != nullptr && parts >= 1 && rows > 0 && experts > 0 && experts <= kMostExperts && top > 0 &&
+                  top <= experts && top <= kMostTop && (top < kMostTop || always < 0),
+              "moe_route_sort: %d rows, %d experts, %d chosen", rows, experts, top);
+  LYP_REQUIRE(E >= experts && E <= kMostExperts && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128),
+              "moe_route_sort: %d matrices, tiles of %d rows", E, tile_rows);
+  const size_t lds = sizeof(int32_t) * (3 * E + 1 + kSortWaves * E);
+  moe_sort_kernel<<<1, kSortThreads, lds, stream>>>(idx, pairs, E, tile_rows, expert_off, sorted_pair, place_of,
+                                                    tile_expert, tile_row0, n_tiles,
+                                                    RouteFirst{part, bias, wgt, parts, rows, experts, top, always});
+  LYP_LAUNCH_CHECK("moe_route_sort");
   return 0;
 }
 

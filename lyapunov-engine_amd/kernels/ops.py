@@ -116,7 +116,10 @@ def core() -> ctypes.CDLL:
         lib.lyp_moe_route.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]
         lib.lyp_moe_route_splits.argtypes = [c_int, c_int]
         lib.lyp_moe_route_fused.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                                            c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]
+                                            c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p]
+        lib.lyp_moe_route_sort.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                                           c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_void_p]
         lib.lyp_moe_tile_rows.argtypes = [c_int, c_int]
         lib.lyp_moe_most_tiles.argtypes = [c_int, c_int, c_int]
         lib.lyp_moe_sort.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -1363,9 +1366,15 @@ def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, top: int, always:
     return idx, wgt
 
 
-def moe_route_from(x: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, top: int, always: int = -1):
+ROUTE_SORT_MAX_ROWS = 64     # steps of up to this many rows choose and sort in one kernel
+
+
+def moe_route_from(x: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | None, top: int, always: int = -1,
+                   sort_for: int = 0):
     """As ``moe_route`` from the router's input: x [T, K] activations, ``router`` [E, K] float; the
-    logits x @ router.T are formed in 32-bit in the same kernel."""
+    logits x @ router.T are formed in 32-bit in the same kernel.  ``sort_for`` > 0 (the number of
+    expert matrices, the always-used one included): also returns the ``MoePlan`` of the choices, as
+    ``moe_sort`` makes it; with few rows the choice and the sort are one kernel."""
     _dev(x, router, bias)
     _f32(router, bias)
     T, K = x.shape
@@ -1379,15 +1388,21 @@ def moe_route_from(x: torch.Tensor, router: torch.Tensor, bias: torch.Tensor | N
     # few rows: several workgroups share the inner dimension and leave partial sums
     splits = lib.lyp_moe_route_splits(T, K)
     part = torch.empty((splits, T, E), dtype=torch.float32, device=x.device) if splits > 1 else None
+    together = sort_for > 0 and splits > 1 and T <= ROUTE_SORT_MAX_ROWS
     _check(lib.lyp_moe_route_fused(_p(x), x.stride(0), _code(x.dtype), _p(router), _p(bias), T, E, K, top, _p(idx),
-                                   _p(wgt), int(always), _p(part), splits, _stream()), lib)
-    return idx, wgt
+                                   _p(wgt), int(always), _p(part), splits, 0 if together else 1, _stream()), lib)
+    if not sort_for:
+        return idx, wgt
+    return idx, wgt, MoePlan(idx, sort_for, route=(part, bias, top, always, wgt) if together else None)
 
 
 class MoePlan:
     """Where the (token, choice) pairs of a step stand once sorted by expert, on the device."""
 
-    def __init__(self, idx: torch.Tensor, E: int):
+    def __init__(self, idx: torch.Tensor, E: int, route=None):
+        """``route`` (partial sums [parts, T, experts], bias, top, always, weights): the choices are not
+        made yet; the sort's kernel adds the router's partial sums up, chooses into ``idx`` and the
+        weights, and sorts."""
         lib = core()
         self.pairs, self.top, self.E = idx.numel(), idx.shape[1], E
         self.tile_rows = lib.lyp_moe_tile_rows(self.pairs, E)
@@ -1400,6 +1415,13 @@ class MoePlan:
             views.append(buf[at:at + n])
             at += n
         self.expert_off, self.sorted_pair, self.place_of, self.tile_expert, self.tile_row0, self.n_tiles = views
+        if route is not None:
+            part, bias, top, always, wgt = route
+            _check(lib.lyp_moe_route_sort(_p(part), part.shape[0], _p(bias), part.shape[1], part.shape[2], top, always,
+                                          _p(idx), _p(wgt), E, self.tile_rows, _p(self.expert_off), _p(self.sorted_pair),
+                                          _p(self.place_of), _p(self.tile_expert), _p(self.tile_row0), _p(self.n_tiles),
+                                          _stream()), lib)
+            return
         _check(lib.lyp_moe_sort(_p(idx), self.pairs, E, self.tile_rows, _p(self.expert_off), _p(self.sorted_pair),
                                 _p(self.place_of), _p(self.tile_expert), _p(self.tile_row0), _p(self.n_tiles),
                                 _stream()), lib)

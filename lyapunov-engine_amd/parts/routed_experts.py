@@ -85,10 +85,10 @@ class RoutedExperts(FeedForward):
         shared expert's and ``addend`` (the other branch's output, activations [T, hidden])."""
         T = x.shape[0]
         always = self.num_experts if self.shared_folded else -1
-        idx, wgt = ops.moe_route_from(x, self.router_f, self.router_bias_f, self.top, always)
+        idx, wgt, plan = ops.moe_route_from(x, self.router_f, self.router_bias_f, self.top, always,
+                                            sort_for=self.gate_up.shape[0])
         if RoutedExperts.choices_log is not None:
             RoutedExperts.choices_log.append(idx[:, :self.top])
-        plan = ops.moe_sort(idx, self.gate_up.shape[0])
         act = ops.moe_gemm(x, self.gate_up, plan, gated=True, limit=self.limit, alpha=self.gate_slope)
         y = ops.moe_gemm(act, self.down, plan, gated=False)
         shared = None

@@ -390,7 +390,8 @@ def test_pairs_sorted_by_expert_in_their_own_order(shape):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(1, 5, 2, 72, 40, 28), (7, 5, 2, 72, 40, 0), (300, 3, 3, 64, 20, 16), (40, 70, 5, 48, 8, 24),
                                    (700, 4, 1, 100, 52, 0), (33, 16, 4, 192, 96, 64), (9, 6, 2, 64, 48, 48),
-                                   (900, 6, 2, 64, 48, 48), (70, 130, 3, 40, 16, 0), (600, 3, 2, 256, 512, 0), (600, 2, 1, 512, 512, 512)])
+                                   (900, 6, 2, 64, 48, 48), (70, 130, 3, 40, 16, 0), (600, 3, 2, 256, 512, 0), (600, 2, 1, 512, 512, 512),
+                                   (5, 12, 3, 512, 64, 0), (40, 7, 2, 1024, 32, 32)])    # few rows of a wide model: choice and sort in one kernel
 def test_routed_experts_against_the_plain_mixture(dtype, shape):
     """The whole feed-forward part, with another branch's output added in, for steps of one token,
     of few and of many (tiles of 16 and of 64 rows), sizes without 16-byte rows among them, and a
