@@ -863,11 +863,11 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
               "moe_gemm: bad sizes N=%d K=%d lda=%d ldw=%d ldo=%d", N, K, lda, ldw, ldo);
   LYP_REQUIRE(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "moe_gemm: tiles of %d rows", tile_rows);
   if (most_tiles == 0) return 0;
-  // with tiles of 128 rows: 256 matrix rows a tile (gated: 128 output columns) where there are that many columns
-  // (measured on 8,192 pairs, 32 experts of 1,536 x 2,048: 237 / 159 us against 225 / 150 us for the
-  // four-wave tile, which leaves room for two workgroups a compute unit)
-  const bool big = false;
-  const int tile_cols = tile_rows != 128 ? 64 : (big ? (gated ? 128 : 256) : (gated ? 64 : 128));
+  // Tiles of 128 rows take 128 matrix rows (gated: 64 output columns).  The kernel's eight-wave form
+  // with 256 matrix rows was measured and is not used: on 8,192 pairs and 32 experts of 1,536 x 2,048
+  // 237 / 159 us against 225 / 150 us for the four-wave tile, which leaves room for two workgroups a
+  // compute unit.
+  const int tile_cols = tile_rows != 128 ? 64 : (gated ? 64 : 128);
   const int col_tiles = (N + tile_cols - 1) / tile_cols;
   LYP_REQUIRE(col_tiles <= 65535, "moe_gemm: too many columns for one launch");
   const int esz = dtype == kF32 ? 4 : 2;
@@ -891,10 +891,7 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
       tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok)
 #define LYP_MOE_T(T)                                 \
   do {                                               \
-    if (tile_rows == 128 && big) {                   \
-      if (gated) { LYP_MOE_WIDE(T, true, 8); }       \
-      else { LYP_MOE_WIDE(T, false, 8); }            \
-    } else if (tile_rows == 128) {                   \
+    if (tile_rows == 128) {                          \
       if (gated) { LYP_MOE_WIDE(T, true, 4); }       \
       else { LYP_MOE_WIDE(T, false, 4); }            \
     } else if (tile_rows == 64) {                    \
