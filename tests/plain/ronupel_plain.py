@@ -97,9 +97,9 @@ def expert(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Te
 
 
 def route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor, top: int, chosen: torch.Tensor | None = None):
-    """-> (experts [n, top], weights [n, top], margin [n]): the ``top`` largest of W_router h + bias,
-    and the softmax over those alone; the margin is what the last chosen logit has over the first
-    one left out.  With ``chosen`` the choice is given (another run's, where the two must route
+    """-> (experts [n, top], weights [n, top], margin [n], size [n]): the ``top`` largest of
+    W_router h + bias, and the softmax over those alone; the margin is what the last chosen logit has
+    over the first one left out, the size the largest logit's magnitude.  With ``chosen`` the choice is given (another run's, where the two must route
     alike to be compared) and only the weights are worked out."""
     z = h @ router.T + bias
     srt = torch.sort(z, dim=-1, descending=True).values
@@ -109,15 +109,15 @@ def route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor, top: int, c
     else:
         idx = chosen.long()
         val = torch.gather(z, 1, idx)
-    return idx, torch.softmax(val, dim=-1), margin
+    return idx, torch.softmax(val, dim=-1), margin, z.abs().max(-1).values
 
 
 def moe(h: torch.Tensor, w: dict, mlp: dict, chosen: torch.Tensor | None = None, notes: dict | None = None) -> torch.Tensor:
     """``w``: the feed-forward's tensors by short name (router, router.b, e<j>.gate/up/down,
     shared.gate/up/down).  ``notes`` receives the choice and its margin."""
-    idx, wt, margin = route(h, w["router"], w["router.b"], int(mlp["router"]["top"]), chosen)
+    idx, wt, margin, size = route(h, w["router"], w["router.b"], int(mlp["router"]["top"]), chosen)
     if notes is not None:
-        notes.update(chosen=idx, margin=margin)
+        notes.update(chosen=idx, margin=margin, size=size)
     out = torch.zeros_like(h)
     limit = float(mlp["expert"]["limit"])
     for t in range(h.shape[0]):

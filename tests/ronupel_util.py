@@ -136,10 +136,11 @@ class RouterLog:
         return {rid: [torch.cat(p) for p in per] if per and per[0] else [] for rid, per in out.items()}
 
 
-def plain_logits_routed_alike(folder: str, requests: dict, chosen: dict, clear: float = 0.5) -> dict:
+def plain_logits_routed_alike(folder: str, requests: dict, chosen: dict, clear: float = 0.1) -> dict:
     """As ``plain_logits`` with the experts the engine chose.  A 16-bit run may decide a close call
     the other way, which says nothing about its kernels; what it must not do is choose otherwise
-    where the plain model's margin is clear: that is asserted here."""
+    where the plain model's margin is clear (more than ``clear`` of the token's largest router logit, and
+    more than 0.5): that is asserted here."""
     if folder not in _PLAIN:
         _PLAIN[folder] = RP.load(folder)
     cfg, tensors = _PLAIN[folder]
@@ -153,7 +154,7 @@ def plain_logits_routed_alike(folder: str, requests: dict, chosen: dict, clear: 
             differs = (torch.sort(theirs.long(), -1).values != torch.sort(nf["chosen"], -1).values).any(-1)
             if differs.any():
                 first = int(torch.nonzero(differs)[0])      # later tokens follow another history
-                assert float(nf["margin"][first]) < clear, (f"request {rid!r}, routed layer run {run}, position {first}: "
+                assert float(nf["margin"][first]) < max(0.5, clear * float(nf["size"][first])), (f"request {rid!r}, routed layer run {run}, position {first}: "
                                                             f"the engine chose {theirs[first].tolist()}, the plain model "
                                                             f"{nf['chosen'][first].tolist()} with a margin of {float(nf['margin'][first]):.3f}")
                 break

@@ -77,11 +77,11 @@ def test_router_takes_the_largest_and_weighs_them_alone():
     h = torch.eye(4, dtype=F64)[:1]
     router = torch.tensor([[1.0, 0, 0, 0], [3.0, 0, 0, 0], [2.0, 0, 0, 0], [-1.0, 0, 0, 0]], dtype=F64)
     bias = torch.tensor([0.0, 0.0, 0.0, 3.5], dtype=F64)
-    idx, w, margin = RP.route(h, router, bias, 2)
+    idx, w, margin, size = RP.route(h, router, bias, 2)
     assert idx[0].tolist() == [1, 3]                                       # 3.0 and -1 + 3.5
-    assert margin.tolist() == pytest.approx([0.5])                         # 2.5 chosen last, 2.0 the first left out
+    assert margin.tolist() == pytest.approx([0.5]) and size.tolist() == [3.0]   # 2.5 chosen last, 2.0 the first left out
     assert w[0].tolist() == pytest.approx([1 / (1 + math.exp(-0.5)), 1 / (1 + math.exp(0.5))])
-    idx, w, _ = RP.route(h, router, bias, 2, chosen=torch.tensor([[0, 2]]))
+    idx, w, _, _ = RP.route(h, router, bias, 2, chosen=torch.tensor([[0, 2]]))
     assert idx[0].tolist() == [0, 2] and w[0].tolist() == pytest.approx([1 / (1 + math.e), math.e / (1 + math.e)])
 
 

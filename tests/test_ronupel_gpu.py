@@ -179,6 +179,24 @@ def test_long_decoding_past_every_window(folders, name):
     check(t, run(folders, name, dtype, t), folders, name, dtype, "long decoding")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_far_keys_and_windows_longer_than_a_partition(tmp_path, dtype):
+    """1,300 tokens through a layer that sees everything (keys a thousand tokens back, in a prompt's
+    portion and for single tokens, in several partitions) and one whose window of 300 spans
+    partitions and keeps 33 first tokens; portions that end inside pages and tiles."""
+    cfg = config(211, 96, [attn(4, 2, 32, 32, dims=16, base=5000.0, factor=2.0, scale=0.35, mlp=moe(6, 2, 40, 3.0, shared=(40, 3.0))),
+                           attn(2, 1, 64, 64, window=300, keep=33, dims=64, scale=0.25, mlp=moe(3, 1, 24, 1.0))],
+                 loop=(0, 2, 2))
+    folder = write_model(str(tmp_path / "m"), cfg, seed=13, dtype=dtype)
+    toks = random_tokens(1300, 211, seed=6)
+    t = Trace({"x": toks})
+    for n in (511, 3, 258, 490):
+        t.step([("x", n)], want="last")
+    for _ in range(38):
+        t.step([("x", 1)])
+    check_folder(t, run_folder(folder, dtype, t, block_size=16), folder, dtype, "far keys")
+
+
 def test_windowed_layers_give_pages_back_and_keep_the_first(folders):
     """A model whose layers are all windowed runs a request far longer than its pool: pages behind
     the window return, those of the kept first tokens stay."""
