@@ -497,14 +497,15 @@ template <typename T, int NW>
 struct MoeWide {
   static constexpr int kKT = 128 / sizeof(T);
   static constexpr int kLD = kKT + (sizeof(T) == 2 ? 8 : 4);
-  static constexpr int kBRows = 32 * NW;                             // matrix rows a tile: 128 or 256
+  static constexpr int kBRows = 128;                                 // matrix rows a tile
   static constexpr int kBytes = 2 * (128 + kBRows) * kLD * sizeof(T);   // both buffers
 };
 
-// The same product for many rows an expert: tiles of 128 rows and 32 NW matrix rows (GATED: half of
-// them gate columns, half their up columns), NW = 4 or 8 waves in 2 x NW / 2, a wave 64 rows x 2
-// blocks of 32 matrix rows on the 32x32 instruction, so that a fragment read from LDS feeds two
-// products.  The larger tile reads a third less per product from the second-level cache.
+// The same product for many rows an expert: tiles of 128 rows and 128 matrix rows (GATED: 64 gate
+// columns and their 64 up columns) on the 32x32 instruction.  NW = 4 waves in 2 x 2: a wave takes two
+// blocks of 32 rows x two blocks of 32 matrix rows, so that a fragment read from LDS feeds two
+// products.  NW = 8 waves in 4 x 2: a wave takes one block of rows x two blocks of matrix rows: half
+// the sums a wave, twice the waves a compute unit to fill each other's waits.
 template <typename T, bool GATED, int NW>
 __global__ __launch_bounds__(NW * 64) void moe_gemm_wide_kernel(
     const T* __restrict__ a, int lda, const T* __restrict__ w, long long w_expert_stride, int ldw,
@@ -543,11 +544,13 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_wide_kernel(
   const int c0 = (work / static_cast<int>(gridDim.x)) * TN;
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int wm = wave % 2, wn = wave / 2;
-  // this wave's two blocks of 32 rows: wm and wm + 2, so that a tile whose last rows are missing
+  constexpr int RB = 8 / NW;           // blocks of 32 rows a wave: 2 or 1
+  constexpr int WM = 4 / RB;           // waves side by side over the tile's rows
+  const int wm = wave % WM, wn = wave / WM;
+  // this wave's blocks of 32 rows: wm (and wm + 2), so that a tile whose last rows are missing
   // (an expert's tail) leaves every wave with less to do, not some with nothing
-  const int rb[2] = {wm, wm + 2};
-  const bool rb_live[2] = {row0 + rb[0] * 32 < row_end, row0 + rb[1] * 32 < row_end};
+  const int rb[2] = {wm, wm + WM};
+  const bool rb_live[2] = {row0 + rb[0] * 32 < row_end, RB > 1 && row0 + rb[1] * 32 < row_end};
   const T* we = w + static_cast<size_t>(e) * w_expert_stride;
 
   const T* a_src[A_PER];
@@ -609,9 +612,9 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_wide_kernel(
   };
   // this wave: row blocks rb[0], rb[1]; matrix-row blocks fb[0], fb[1] of the tile
   const int fb[2] = {GATED ? wn * 32 : wn * 64, GATED ? BROWS / 2 + wn * 32 : wn * 64 + 32};
-  f32x16 acc[2][2];
+  f32x16 acc[RB][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < RB; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -623,14 +626,14 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_wide_kernel(
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       const int kk = s * 2 * MW::kElems + (lane / 32) * MW::kElems;
-      typename MW::Frag xf[2], wf[2];
+      typename MW::Frag xf[RB], wf[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < RB; ++i)
         if (rb_live[i]) xf[i] = *reinterpret_cast<const typename MW::Frag*>(As + (rb[i] * 32 + lane % 32) * LD + kk);
-        wf[i] = *reinterpret_cast<const typename MW::Frag*>(Bs + (fb[i] + lane % 32) * LD + kk);
-      }
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int j = 0; j < 2; ++j) wf[j] = *reinterpret_cast<const typename MW::Frag*>(Bs + (fb[j] + lane % 32) * LD + kk);
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
         if (!rb_live[i]) continue;
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = MW::mma(wf[j], xf[i], acc[i][j]);
@@ -657,7 +660,7 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_wide_kernel(
 
   // register v of lane l: matrix row 8 * (v / 4) + 4 * (l / 32) + v % 4 of the block, token l % 32
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < RB; ++i) {
     const int place = row0 + rb[i] * 32 + lane % 32;
     if (place >= row_end) continue;
     T* orow = out + static_cast<size_t>(place) * ldo;
@@ -863,10 +866,10 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
               "moe_gemm: bad sizes N=%d K=%d lda=%d ldw=%d ldo=%d", N, K, lda, ldw, ldo);
   LYP_REQUIRE(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "moe_gemm: tiles of %d rows", tile_rows);
   if (most_tiles == 0) return 0;
-  // Tiles of 128 rows take 128 matrix rows (gated: 64 output columns).  The kernel's eight-wave form
-  // with 256 matrix rows was measured and is not used: on 8,192 pairs and 32 experts of 1,536 x 2,048
-  // 237 / 159 us against 225 / 150 us for the four-wave tile, which leaves room for two workgroups a
-  // compute unit.
+  // Tiles of 128 rows take 128 matrix rows (gated: 64 output columns), eight waves a tile.  Measured
+  // on 8,192 pairs and 32 experts of 1,536 x 2,048 (gated / down, the kernels alone): four waves a tile
+  // 242 / 162 us, eight waves 221 / 146 us, eight waves with rounds of 64 bytes a row 255 / 168 us; a
+  // tile of 256 matrix rows with eight waves (one workgroup a compute unit) was slower than either.
   const int tile_cols = tile_rows != 128 ? 64 : (gated ? 64 : 128);
   const int col_tiles = (N + tile_cols - 1) / tile_cols;
   LYP_REQUIRE(col_tiles <= 65535, "moe_gemm: too many columns for one launch");
@@ -892,8 +895,8 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
 #define LYP_MOE_T(T)                                 \
   do {                                               \
     if (tile_rows == 128) {                          \
-      if (gated) { LYP_MOE_WIDE(T, true, 4); }       \
-      else { LYP_MOE_WIDE(T, false, 4); }            \
+      if (gated) { LYP_MOE_WIDE(T, true, 8); }       \
+      else { LYP_MOE_WIDE(T, false, 8); }            \
     } else if (tile_rows == 64) {                    \
       if (gated) LYP_MOE(T, 4, true);                \
       else LYP_MOE(T, 4, false);                     \
