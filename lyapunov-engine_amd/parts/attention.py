@@ -89,6 +89,38 @@ class AttentionWork(StepPlanner):
 _WORK = AttentionWork()
 
 
+# The launch shapes of the two attention kernels for a step, from the planner's host values alone
+# (no device work: a test can check them against the kernels' index ranges).  Any mixer that keeps
+# its keys and values in ``PagedSpec.keys_and_values`` pages launches the kernels by these.
+def prefill_launch(meta: dict, dtype: torch.dtype, page_size: int, *, num_heads: int, num_kv_heads: int, head_dim: int,
+                   window: int = 0) -> Optional[dict]:
+    """For the tiles of requests that bring several tokens: in how many runs every tile's keys
+    are cut, whether workgroups pair a light tile with a heavy one, and the floats of the
+    workspaces the runs' partial results need.  None: no tiles."""
+    n_tiles = meta["n_tiles"]
+    if not n_tiles:
+        return None
+    # Tiles come in rising order of the keys they see; when the first sees less than half
+    # of what the last does, a workgroup may take one from each end.
+    few, many = (min(k, window + 64) if window else k for k in meta["tile_keys"])
+    # few new tokens over many keys: the keys in runs, for workgroups of their own
+    parts = ops.attn_prefill_plan(n_tiles, many, num_heads, num_kv_heads, head_dim, dtype, page_size)
+    n = n_tiles * PREFILL_TILE * num_heads * parts if parts > 1 else 0
+    return dict(n_tiles=n_tiles, parts=parts, pair=2 * few <= many, part_o=n * head_dim, part_ml=n * 2)
+
+
+def decode_launch(meta: dict, *, num_heads: int, num_kv_heads: int, head_dim: int) -> Optional[dict]:
+    """For the requests that bring one token: keys per workgroup, the most partitions a
+    request can have, and the floats of the partitions' workspaces.  None: no such request."""
+    n_dec, max_ctx = meta["n_dec"], meta["max_ctx_dec"]
+    if not n_dec:
+        return None
+    part = ops.attn_decode_plan(n_dec, max_ctx, num_heads, num_kv_heads, head_dim)
+    max_parts = max(1, (max_ctx + part - 1) // part)
+    n = n_dec * num_heads * max_parts
+    return dict(n_dec=n_dec, part_keys=part, max_parts=max_parts, part_o=n * head_dim, part_ml=n * 2)
+
+
 @MIXERS.register("paged_attention")
 class PagedAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -127,33 +159,12 @@ class PagedAttention(Mixer):
     def step_planner(self):
         return _WORK
 
-    # The launch shapes of the two attention kernels for a step, from the planner's host values
-    # alone (no device work: a test can check them against the kernels' index ranges).
     def prefill_launch(self, meta: dict, dtype: torch.dtype, page_size: int) -> Optional[dict]:
-        """For the tiles of requests that bring several tokens: in how many runs every tile's keys
-        are cut, whether workgroups pair a light tile with a heavy one, and the floats of the
-        workspaces the runs' partial results need.  None: no tiles."""
-        n_tiles = meta["n_tiles"]
-        if not n_tiles:
-            return None
-        # Tiles come in rising order of the keys they see; when the first sees less than half
-        # of what the last does, a workgroup may take one from each end.
-        few, many = (min(k, self.window + 64) if self.window else k for k in meta["tile_keys"])
-        # few new tokens over many keys: the keys in runs, for workgroups of their own
-        parts = ops.attn_prefill_plan(n_tiles, many, self.num_heads, self.num_kv_heads, self.head_dim, dtype, page_size)
-        n = n_tiles * PREFILL_TILE * self.num_heads * parts if parts > 1 else 0
-        return dict(n_tiles=n_tiles, parts=parts, pair=2 * few <= many, part_o=n * self.head_dim, part_ml=n * 2)
+        return prefill_launch(meta, dtype, page_size, num_heads=self.num_heads, num_kv_heads=self.num_kv_heads,
+                              head_dim=self.head_dim, window=self.window)
 
     def decode_launch(self, meta: dict) -> Optional[dict]:
-        """For the requests that bring one token: keys per workgroup, the most partitions a
-        request can have, and the floats of the partitions' workspaces.  None: no such request."""
-        n_dec, max_ctx = meta["n_dec"], meta["max_ctx_dec"]
-        if not n_dec:
-            return None
-        part = ops.attn_decode_plan(n_dec, max_ctx, self.num_heads, self.num_kv_heads, self.head_dim)
-        max_parts = max(1, (max_ctx + part - 1) // part)
-        n = n_dec * self.num_heads * max_parts
-        return dict(n_dec=n_dec, part_keys=part, max_parts=max_parts, part_o=n * self.head_dim, part_ml=n * 2)
+        return decode_launch(meta, num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, head_dim=self.head_dim)
 
     takes_pending_norm = True   # x may be an ops.PendingNorm: the q/k/v product norms on its way in
 

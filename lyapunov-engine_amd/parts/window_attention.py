@@ -30,7 +30,7 @@ import torch
 from ..config.registry import MIXERS, POSITION_ENCODINGS
 from ..config.specs import PartSpec
 from ..kernels import ops
-from .attention import AttentionWork, PagedAttention
+from .attention import AttentionWork, decode_launch, prefill_launch
 from .base import LayerCache, Mixer, PagedSpec, StepContext, WeightSource, WeightSpec
 
 _WORK = AttentionWork()
@@ -58,9 +58,6 @@ class SinkWindowAttention(Mixer):
         self.names = n
         # equal key and value sizes in multiples of 16: the matrix-core kernels
         self.matrix_cores = self.dim == self.vdim and self.dim % 16 == 0 and self.dim <= 256
-        self._planner = PagedAttention.__new__(PagedAttention)   # the launch shapes of those kernels, for these sizes
-        self._planner.num_heads, self._planner.num_kv_heads = self.num_heads, self.num_kv_heads
-        self._planner.head_dim, self._planner.window = self.dim, self.window
         self.qkv_proj = self.o_proj = self.q_norm = self.k_norm = self.sink = None
         self.q_norm_f = self.k_norm_f = self.sink_f = None
 
@@ -113,7 +110,8 @@ class SinkWindowAttention(Mixer):
         common = dict(num_heads=H, num_kv_heads=G, head_dim=self.dim, window=self.window, scale=self.scale,
                       keep_first=self.keep_first, sink=self.sink_f)
         work = ctx.plans[AttentionWork.key]
-        pre = self._planner.prefill_launch(work.meta, ctx.dtype, g.page_size)
+        sizes = dict(num_heads=H, num_kv_heads=G, head_dim=self.dim)
+        pre = prefill_launch(work.meta, ctx.dtype, g.page_size, window=self.window, **sizes)
         if pre is not None:
             part_o = part_ml = None
             if pre["parts"] > 1:
@@ -122,7 +120,7 @@ class SinkWindowAttention(Mixer):
             ops.attn_prefill(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len,
                              work.arrays["tile_seq"], work.arrays["tile_q0"], pre["n_tiles"], pair=pre["pair"],
                              parts=pre["parts"], part_o=part_o, part_ml=part_ml, **common)
-        dec = self._planner.decode_launch(work.meta)
+        dec = decode_launch(work.meta, **sizes)
         if dec is not None:
             part_o = ctx.scratch("attn_part_o", dec["part_o"])
             part_ml = ctx.scratch("attn_part_ml", dec["part_ml"])
