@@ -342,7 +342,8 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
 // ------------------------------------------------------------------- product
 // grid (most tiles, column tiles); 256 threads.  MB 16-row blocks of rows and
 // 64 output columns per workgroup; a wave takes one row block and 4 / (4 / MB)
-// column blocks (MB = 4), or the one row block and one column block (MB = 1).
+// column blocks (MB = 4, tiles of 64 rows; MB = 1 would be one row block and one
+// column block a wave: tiles of 16 rows take moe_gemm_few_kernel instead).
 template <typename T, int MB, bool GATED, typename TO>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(
     const T* __restrict__ a, int lda, const T* __restrict__ w, long long w_expert_stride, int ldw,
@@ -490,6 +491,93 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
       }
       orow[col + i] = from_f32<TO>(y);
     }
+  }
+}
+
+// The same product for launches of few tiles (a decode step: a handful of pairs, each expert's matrix
+// read for one or two rows).  A workgroup takes a tile of up to 16 rows and only 16 output columns
+// (GATED: 16 gate rows and their 16 up rows of the matrix), so that there are many workgroups to pull
+// the matrices through; its four waves share the inner dimension, step by step in turn, take their
+// operands straight from memory into the matrix instruction's registers, four steps' loads in flight,
+// and add their sums up through LDS in the order of the waves.
+constexpr int kFewAhead = 4;
+
+template <typename T, bool GATED>
+__global__ __launch_bounds__(256) void moe_gemm_few_kernel(
+    const T* __restrict__ a, int lda, const T* __restrict__ w, long long w_expert_stride, int ldw,
+    T* __restrict__ out, int ldo, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
+    const int32_t* __restrict__ n_tiles, const int32_t* __restrict__ expert_off,
+    const int32_t* __restrict__ sorted_pair, int top, int N, int K, int up_offset, float limit, float alpha,
+    int vec_ok) {
+  using MW = Mma16Wide<T>;
+  constexpr int KE = MW::kElems, STEP = 4 * KE;
+  __shared__ float s_red[4][2][kWave][4];
+  const int tile = blockIdx.x;
+  if (tile >= n_tiles[0]) return;
+  const int e = tile_expert[tile];
+  const int row0 = tile_row0[tile];
+  const int row_end = expert_off[e + 1];
+  const int c0 = blockIdx.y * 16;
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int r = lane % 16, grp = lane / 16;
+  const T* we = w + static_cast<size_t>(e) * w_expert_stride;
+  const int place = row0 + r;
+  const T* x_row = nullptr;
+  if (place < row_end) x_row = a + static_cast<size_t>(GATED ? sorted_pair[place] / top : place) * lda;
+  const int col = c0 + r;
+  const T* g_row = col < N ? we + static_cast<size_t>(col) * ldw : nullptr;
+  const T* u_row = GATED && col < N ? we + static_cast<size_t>(col + up_offset) * ldw : nullptr;
+  auto fetch = [&](const T* src, int k) {
+    typename MW::Frag f;
+#pragma unroll
+    for (int i = 0; i < KE; ++i) f[i] = from_f32<T>(0.f);
+    if (src != nullptr) {
+      if (vec_ok && k + KE <= K) {
+        f = *reinterpret_cast<const typename MW::Frag*>(src + k);
+      } else {
+#pragma unroll
+        for (int i = 0; i < KE; ++i)
+          if (k + i < K) f[i] = src[k + i];
+      }
+    }
+    return f;
+  };
+  f32x4 acc_g = f32x4{0.f, 0.f, 0.f, 0.f}, acc_u = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int steps = (K + STEP - 1) / STEP;
+  for (int s0 = wave; s0 < steps; s0 += 4 * kFewAhead) {
+    typename MW::Frag xf[kFewAhead], gf[kFewAhead], uf[kFewAhead];
+#pragma unroll
+    for (int t = 0; t < kFewAhead; ++t) {
+      const int k = (s0 + 4 * t) * STEP + grp * KE;      // beyond K: zeros
+      xf[t] = fetch(x_row, k);
+      gf[t] = fetch(g_row, k);
+      if constexpr (GATED) uf[t] = fetch(u_row, k);
+    }
+#pragma unroll
+    for (int t = 0; t < kFewAhead; ++t) {
+      acc_g = MW::mma(gf[t], xf[t], acc_g);
+      if constexpr (GATED) acc_u = MW::mma(uf[t], xf[t], acc_u);
+    }
+  }
+  *reinterpret_cast<f32x4*>(&s_red[wave][0][lane][0]) = acc_g;
+  if constexpr (GATED) *reinterpret_cast<f32x4*>(&s_red[wave][1][lane][0]) = acc_u;
+  __syncthreads();
+  if (wave != 0 || place >= row_end) return;
+  // lane l: token row l % 16, features c0 + 4 * (l / 16) + {0..3}
+  T* orow = out + static_cast<size_t>(place) * ldo;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = c0 + 4 * grp + i;
+    if (c >= N) continue;
+    float y = s_red[0][0][lane][i] + s_red[1][0][lane][i] + s_red[2][0][lane][i] + s_red[3][0][lane][i];
+    if constexpr (GATED) {
+      const float up = s_red[0][1][lane][i] + s_red[1][1][lane][i] + s_red[2][1][lane][i] + s_red[3][1][lane][i];
+      const float g = fminf(y, limit);
+      const float u = fminf(fmaxf(up, -limit), limit);
+      y = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    }
+    orow[c] = from_f32<T>(y);
   }
 }
 
@@ -871,7 +959,12 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
   // 242 / 162 us, eight waves 221 / 146 us, eight waves with rounds of 64 bytes a row 255 / 168 us; a
   // tile of 256 matrix rows with eight waves (one workgroup a compute unit) was slower than either.
   const int tile_cols = tile_rows != 128 ? 64 : (gated ? 64 : 128);
-  const int col_tiles = (N + tile_cols - 1) / tile_cols;
+  // tiles of 16 rows (few rows an expert: a decode step's, a short portion's) are 16 columns wide, so
+  // that the launch has workgroups enough to pull the matrices through (one token that chooses 4 of 32
+  // experts of 1,536 x 2,048: 37 / 23 us with tiles of 64 columns through LDS, 15 / 9.5 us so; eight
+  // tokens: 64 / 33 us against 53 / 30 us)
+  const bool few = tile_rows == 16;
+  const int col_tiles = few ? (N + 15) / 16 : (N + tile_cols - 1) / tile_cols;
   LYP_REQUIRE(col_tiles <= 65535, "moe_gemm: too many columns for one launch");
   const int esz = dtype == kF32 ? 4 : 2;
   const int vec = 16 / esz;
@@ -892,23 +985,28 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
   moe_gemm_wide_kernel<T, G, NWV><<<grid, NWV * 64, MoeWide<T, NWV>::kBytes, stream>>>(                         \
       static_cast<const T*>(a), lda, static_cast<const T*>(w), w_expert_stride, ldw, static_cast<T*>(out), ldo, \
       tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok)
+#define LYP_MOE_FEW(T, G)                                                                                       \
+  moe_gemm_few_kernel<T, G><<<grid, 256, 0, stream>>>(                                                          \
+      static_cast<const T*>(a), lda, static_cast<const T*>(w), w_expert_stride, ldw, static_cast<T*>(out), ldo, \
+      tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok)
 #define LYP_MOE_T(T)                                 \
   do {                                               \
-    if (tile_rows == 128) {                          \
+    if (few) {                                       \
+      if (gated) LYP_MOE_FEW(T, true);               \
+      else LYP_MOE_FEW(T, false);                    \
+    } else if (tile_rows == 128) {                   \
       if (gated) { LYP_MOE_WIDE(T, true, 8); }       \
       else { LYP_MOE_WIDE(T, false, 8); }            \
-    } else if (tile_rows == 64) {                    \
+    } else {                                         \
       if (gated) LYP_MOE(T, 4, true);                \
       else LYP_MOE(T, 4, false);                     \
-    } else {                                         \
-      if (gated) LYP_MOE(T, 1, true);                \
-      else LYP_MOE(T, 1, false);                     \
     }                                                \
   } while (0)
   if (dtype == kF32) LYP_MOE_T(float);
   else if (dtype == kBF16) LYP_MOE_T(bf16_t);
   else LYP_REQUIRE(false, "moe_gemm: unknown dtype %d", dtype);
 #undef LYP_MOE_T
+#undef LYP_MOE_FEW
 #undef LYP_MOE_WIDE
 #undef LYP_MOE
   LYP_LAUNCH_CHECK("moe_gemm");
