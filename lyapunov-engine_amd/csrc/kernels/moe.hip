@@ -9,7 +9,8 @@
 //              the pairs, whatever the timing.  Nothing goes back to the host: the
 //              products' grids are sized for the most tiles there can be.
 //   product    a tile of one expert's rows times a tile of that expert's matrix,
-//              on the matrix cores, through LDS.  GATED: rows are gathered from
+//              on the matrix cores (through LDS for many rows an expert, straight
+//              from memory for few).  GATED: rows are gathered from
 //              the step's activations by token, the gate's and the up
 //              projection's columns are computed side by side and the epilogue
 //              writes  min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1).
@@ -340,162 +341,12 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
 }
 
 // ------------------------------------------------------------------- product
-// grid (most tiles, column tiles); 256 threads.  MB 16-row blocks of rows and
-// 64 output columns per workgroup; a wave takes one row block and 4 / (4 / MB)
-// column blocks (MB = 4, tiles of 64 rows; MB = 1 would be one row block and one
-// column block a wave: tiles of 16 rows take moe_gemm_few_kernel instead).
-template <typename T, int MB, bool GATED, typename TO>
-__global__ __launch_bounds__(256) void moe_gemm_kernel(
-    const T* __restrict__ a, int lda, const T* __restrict__ w, long long w_expert_stride, int ldw,
-    TO* __restrict__ out, int ldo, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
-    const int32_t* __restrict__ n_tiles, const int32_t* __restrict__ expert_off,
-    const int32_t* __restrict__ sorted_pair, int top, int N, int K, int up_offset, float limit, float alpha,
-    int vec_ok) {
-  using MW = Mma16Wide<T>;
-  constexpr int VEC = 16 / sizeof(T);
-  constexpr int KT = 128 / sizeof(T);                 // inner values a round: 128 bytes of every row
-  constexpr int LD = KT + (sizeof(T) == 2 ? 8 : 4);   // padded row: 16-byte reads of 16 rows fall into distinct banks
-  constexpr int TM = 16 * MB, TN = 64;
-  constexpr int BROWS = GATED ? 2 * TN : TN;
-  constexpr int WM = MB, WN = 4 / MB, CB = 4 / WN;
-  constexpr int STEPS = KT / (4 * MW::kElems);
-  constexpr int A_PER = (TM * KT / VEC + 255) / 256, B_PER = (BROWS * KT / VEC + 255) / 256;
-  typedef T VecT __attribute__((ext_vector_type(VEC)));
-  // two buffers: the next round's tiles are written while this round's are read, one barrier a round
-  __shared__ __attribute__((aligned(16))) T As2[2][TM * LD];
-  __shared__ __attribute__((aligned(16))) T Bs2[2][BROWS * LD];
-
-  const int tile = blockIdx.x;
-  if (tile >= n_tiles[0]) return;
-  const int e = tile_expert[tile];
-  const int row0 = tile_row0[tile];
-  const int row_end = expert_off[e + 1];
-  const int c0 = blockIdx.y * TN;
-  const int tid = threadIdx.x, lane = tid % kWave;
-  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int wm = wave % WM, wn = wave / WM;
-  const T* we = w + static_cast<size_t>(e) * w_expert_stride;
-
-  // where this thread's pieces of the two tiles come from
-  const T* a_src[A_PER];
-  int a_k[A_PER], a_lds[A_PER];
-#pragma unroll
-  for (int n = 0; n < A_PER; ++n) {
-    const int v = tid + n * 256;
-    const int r = v / (KT / VEC), kc = (v % (KT / VEC)) * VEC;
-    a_k[n] = kc;
-    a_lds[n] = r * LD + kc;
-    a_src[n] = nullptr;
-    if (v < TM * KT / VEC && row0 + r < row_end) {
-      const int place = row0 + r;
-      const int src_row = GATED ? sorted_pair[place] / top : place;
-      a_src[n] = a + static_cast<size_t>(src_row) * lda;
-    }
-    if (v >= TM * KT / VEC) a_lds[n] = -1;
-  }
-  const T* b_src[B_PER];
-  int b_k[B_PER], b_lds[B_PER];
-#pragma unroll
-  for (int n = 0; n < B_PER; ++n) {
-    const int v = tid + n * 256;
-    const int r = v / (KT / VEC), kc = (v % (KT / VEC)) * VEC;
-    b_k[n] = kc;
-    b_lds[n] = v < BROWS * KT / VEC ? r * LD + kc : -1;
-    b_src[n] = nullptr;
-    if (v < BROWS * KT / VEC) {
-      const int col = c0 + r % TN;
-      if (col < N) b_src[n] = we + static_cast<size_t>(col + (GATED && r >= TN ? up_offset : 0)) * ldw;
-    }
-  }
-  auto fetch = [&](const T* src, int k) {
-    VecT x;
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) x[i] = from_f32<T>(0.f);
-    if (src != nullptr) {
-      if (vec_ok && k + VEC <= K) {
-        x = *reinterpret_cast<const VecT*>(src + k);
-      } else {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i)
-          if (k + i < K) x[i] = src[k + i];
-      }
-    }
-    return x;
-  };
-  VecT a_reg[A_PER], b_reg[B_PER];
-  auto load = [&](int k0) {
-#pragma unroll
-    for (int n = 0; n < A_PER; ++n) a_reg[n] = fetch(a_src[n], k0 + a_k[n]);
-#pragma unroll
-    for (int n = 0; n < B_PER; ++n) b_reg[n] = fetch(b_src[n], k0 + b_k[n]);
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int n = 0; n < A_PER; ++n)
-      if (a_lds[n] >= 0) *reinterpret_cast<VecT*>(As2[buf] + a_lds[n]) = a_reg[n];
-#pragma unroll
-    for (int n = 0; n < B_PER; ++n)
-      if (b_lds[n] >= 0) *reinterpret_cast<VecT*>(Bs2[buf] + b_lds[n]) = b_reg[n];
-  };
-
-  f32x4 acc[CB], acc_up[GATED ? CB : 1];
-#pragma unroll
-  for (int c = 0; c < CB; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int c = 0; c < (GATED ? CB : 1); ++c) acc_up[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  load(0);
-  stash(0);
-  __syncthreads();
-  int buf = 0;
-  for (int k0 = 0; k0 < K; k0 += KT) {
-    const bool more = k0 + KT < K;
-    if (more) load(k0 + KT);
-    const T* As = As2[buf];
-    const T* Bs = Bs2[buf];
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const int kk = s * 4 * MW::kElems + (lane / 16) * MW::kElems;
-      const typename MW::Frag xf = *reinterpret_cast<const typename MW::Frag*>(As + (wm * 16 + lane % 16) * LD + kk);
-#pragma unroll
-      for (int c = 0; c < CB; ++c) {
-        const int brow = (wn * CB + c) * 16 + lane % 16;
-        const typename MW::Frag wf = *reinterpret_cast<const typename MW::Frag*>(Bs + brow * LD + kk);
-        acc[c] = MW::mma(wf, xf, acc[c]);
-        if constexpr (GATED) {
-          const typename MW::Frag uf = *reinterpret_cast<const typename MW::Frag*>(Bs + (TN + brow) * LD + kk);
-          acc_up[c] = MW::mma(uf, xf, acc_up[c]);
-        }
-      }
-    }
-    if (more) stash(buf ^ 1);
-    __syncthreads();
-    buf ^= 1;
-  }
-
-  // lane l: token row wm * 16 + l % 16, features (wn * CB + c) * 16 + 4 * (l / 16) + {0..3}
-  const int place = row0 + wm * 16 + lane % 16;
-  if (place >= row_end) return;
-  TO* orow = out + static_cast<size_t>(place) * ldo;
-#pragma unroll
-  for (int c = 0; c < CB; ++c) {
-    const int col = c0 + (wn * CB + c) * 16 + 4 * (lane / 16);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (col + i >= N) continue;
-      float y = acc[c][i];
-      if constexpr (GATED) {
-        const float g = fminf(y, limit);
-        const float u = fminf(fmaxf(acc_up[c][i], -limit), limit);
-        y = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
-      }
-      orow[col + i] = from_f32<TO>(y);
-    }
-  }
-}
-
-// The same product for launches of few tiles (a decode step: a handful of pairs, each expert's matrix
-// read for one or two rows).  A workgroup takes a tile of up to 16 rows and only 16 output columns
+// Two kernels: tiles of up to 16 rows for experts that see few rows (moe_gemm_few_kernel), tiles of
+// 128 rows through LDS on the 32x32 instruction for experts that see many (moe_gemm_wide_kernel).
+// Both read a row's operands over the inner dimension in a fixed order, whatever the row's place.
+//
+// Launches of few tiles (a decode step: a handful of pairs, each expert's matrix read for one or two
+// rows).  A workgroup takes a tile of up to 16 rows and only 16 output columns
 // (GATED: 16 gate rows and their 16 up rows of the matrix), so that there are many workgroups to pull
 // the matrices through; its four waves share the inner dimension, step by step in turn, take their
 // operands straight from memory into the matrix instruction's registers, four steps' loads in flight,
@@ -589,7 +440,7 @@ struct MoeWide {
   static constexpr int kBytes = 2 * (128 + kBRows) * kLD * sizeof(T);   // both buffers
 };
 
-// The same product for many rows an expert: tiles of 128 rows and 128 matrix rows (GATED: 64 gate
+// Many rows an expert: tiles of 128 rows and 128 matrix rows (GATED: 64 gate
 // columns and their 64 up columns) on the 32x32 instruction.  NW = 4 waves in 2 x 2: a wave takes two
 // blocks of 32 rows x two blocks of 32 matrix rows, so that a fragment read from LDS feeds two
 // products.  NW = 8 waves in 4 x 2: a wave takes one block of rows x two blocks of matrix rows: half
@@ -907,14 +758,16 @@ int lyp_moe_route_fused(const void* x, int ldx, int dtype, const float* w, const
 
 // Rows per tile the products had better use for `pairs` pairs over E experts, and the most tiles
 // there can then be (the products' grid).
-int lyp_moe_tile_rows(int pairs, int E) { return pairs >= 96 * E ? 128 : (pairs >= 32 * E ? 64 : 16); }
+// (from 32 rows an expert on the large tile, half empty as it then is, is ahead of four small ones:
+// 512 tokens, 32 experts of 1,536 x 2,048, 4 chosen: 144 / 81 us in tiles of 64 rows, 120 / 73 us so)
+int lyp_moe_tile_rows(int pairs, int E) { return pairs >= 32 * E ? 128 : 16; }
 int lyp_moe_most_tiles(int pairs, int E, int tile_rows) {
   return (pairs + tile_rows - 1) / tile_rows + std::min(E, pairs);
 }
 
 int lyp_moe_sort(const int32_t* idx, int pairs, int E, int tile_rows, int32_t* expert_off, int32_t* sorted_pair,
                  int32_t* place_of, int32_t* tile_expert, int32_t* tile_row0, int32_t* n_tiles, hipStream_t stream) {
-  LYP_REQUIRE(pairs >= 0 && E > 0 && E <= kMostExperts && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128),
+  LYP_REQUIRE(pairs >= 0 && E > 0 && E <= kMostExperts && (tile_rows == 16 || tile_rows == 128),
               "moe_sort: %d pairs, %d experts, tiles of %d rows", pairs, E, tile_rows);
   const size_t lds = sizeof(int32_t) * (3 * E + 1 + kSortWaves * E);
   moe_sort_kernel<<<1, kSortThreads, lds, stream>>>(const_cast<int32_t*>(idx), pairs, E, tile_rows, expert_off,
@@ -934,7 +787,7 @@ int lyp_moe_route_sort(const float* part, int parts, const float* bias, int rows
   LYP_REQUIRE(part != nullptr && parts >= 1 && rows > 0 && experts > 0 && experts <= kMostExperts && top > 0 &&
                   top <= experts && top <= kMostTop && (top < kMostTop || always < 0),
               "moe_route_sort: %d rows, %d experts, %d chosen", rows, experts, top);
-  LYP_REQUIRE(E >= experts && E <= kMostExperts && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128),
+  LYP_REQUIRE(E >= experts && E <= kMostExperts && (tile_rows == 16 || tile_rows == 128),
               "moe_route_sort: %d matrices, tiles of %d rows", E, tile_rows);
   const size_t lds = sizeof(int32_t) * (3 * E + 1 + kSortWaves * E);
   moe_sort_kernel<<<1, kSortThreads, lds, stream>>>(idx, pairs, E, tile_rows, expert_off, sorted_pair, place_of,
@@ -952,13 +805,13 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
                  int K, float limit, float alpha, hipStream_t stream) {
   LYP_REQUIRE(N > 0 && K > 0 && lda >= K && ldw >= K && ldo >= N && top > 0 && most_tiles >= 0,
               "moe_gemm: bad sizes N=%d K=%d lda=%d ldw=%d ldo=%d", N, K, lda, ldw, ldo);
-  LYP_REQUIRE(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "moe_gemm: tiles of %d rows", tile_rows);
+  LYP_REQUIRE(tile_rows == 16 || tile_rows == 128, "moe_gemm: tiles of %d rows", tile_rows);
   if (most_tiles == 0) return 0;
   // Tiles of 128 rows take 128 matrix rows (gated: 64 output columns), eight waves a tile.  Measured
   // on 8,192 pairs and 32 experts of 1,536 x 2,048 (gated / down, the kernels alone): four waves a tile
   // 242 / 162 us, eight waves 221 / 146 us, eight waves with rounds of 64 bytes a row 255 / 168 us; a
   // tile of 256 matrix rows with eight waves (one workgroup a compute unit) was slower than either.
-  const int tile_cols = tile_rows != 128 ? 64 : (gated ? 64 : 128);
+  const int tile_cols = gated ? 64 : 128;
   // tiles of 16 rows (few rows an expert: a decode step's, a short portion's) are 16 columns wide, so
   // that the launch has workgroups enough to pull the matrices through (one token that chooses 4 of 32
   // experts of 1,536 x 2,048: 37 / 23 us with tiles of 64 columns through LDS, 15 / 9.5 us so; eight
@@ -971,10 +824,6 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
   const int vec_ok = lda % vec == 0 && ldw % vec == 0 && w_expert_stride % vec == 0 &&
                      reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
   dim3 grid(most_tiles, col_tiles);
-#define LYP_MOE(T, MB, G)                                                                                       \
-  moe_gemm_kernel<T, MB, G, T><<<grid, 256, 0, stream>>>(                                                       \
-      static_cast<const T*>(a), lda, static_cast<const T*>(w), w_expert_stride, ldw, static_cast<T*>(out), ldo, \
-      tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok)
 #define LYP_MOE_WIDE(T, G, NWV)                                                                                 \
   static bool wide_set_##G##NWV = false;   /* the tiles take more LDS than a kernel gets unasked */             \
   if (!wide_set_##G##NWV) {                                                                                     \
@@ -994,12 +843,9 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
     if (few) {                                       \
       if (gated) LYP_MOE_FEW(T, true);               \
       else LYP_MOE_FEW(T, false);                    \
-    } else if (tile_rows == 128) {                   \
+    } else {                                         \
       if (gated) { LYP_MOE_WIDE(T, true, 8); }       \
       else { LYP_MOE_WIDE(T, false, 8); }            \
-    } else {                                         \
-      if (gated) LYP_MOE(T, 4, true);                \
-      else LYP_MOE(T, 4, false);                     \
     }                                                \
   } while (0)
   if (dtype == kF32) LYP_MOE_T(float);
@@ -1008,7 +854,6 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
 #undef LYP_MOE_T
 #undef LYP_MOE_FEW
 #undef LYP_MOE_WIDE
-#undef LYP_MOE
   LYP_LAUNCH_CHECK("moe_gemm");
   return 0;
 }
