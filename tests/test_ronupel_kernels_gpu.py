@@ -394,7 +394,7 @@ def test_pairs_sorted_by_expert_in_their_own_order(shape):
                                    (5, 12, 3, 512, 64, 0), (40, 7, 2, 1024, 32, 32)])    # few rows of a wide model: choice and sort in one kernel
 def test_routed_experts_against_the_plain_mixture(dtype, shape):
     """The whole feed-forward part, with another branch's output added in, for steps of one token,
-    of few and of many (tiles of 16 and of 64 rows), sizes without 16-byte rows among them, and a
+    of few and of many (tiles of 16 and of 128 rows), sizes without 16-byte rows among them, and a
     shared expert of the routed experts' size and limit (it then rides in their products)."""
     from lyapunov_engine_amd.parts.base import StepContext
     from lyapunov_engine_amd.parts.routed_experts import RoutedExperts
